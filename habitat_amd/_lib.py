@@ -1,0 +1,87 @@
+"""ctypes binding of libhabitat_mi.so (the C ABI in include/habitat_mi.h).
+
+The library is the only compute path: if it is missing this module raises, it
+never falls back to CPU code.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libhabitat_mi.so")
+
+HBT_OK, HBT_EINVAL, HBT_ESPEC, HBT_EHIP, HBT_ENOMEM, HBT_EALIGN, HBT_ESIZE = 0, -1, -2, -3, -4, -5, -6
+ST_OK, ST_ORIGIN_WAVE_ZERO, ST_DEST_WAVE_ZERO, ST_BAD_GAMMA, ST_ZERO_BLOCKS = 0, 1, 2, 3, 4
+
+
+class DeviceSpec(C.Structure):
+    """hbt_device_spec."""
+    _fields_ = [
+        ("compute_major", C.c_int32), ("compute_minor", C.c_int32),
+        ("max_threads_per_block", C.c_int32), ("max_threads_per_sm", C.c_int32),
+        ("regs_per_block", C.c_int32), ("regs_per_sm", C.c_int32),
+        ("warp_size", C.c_int32), ("num_sms", C.c_int32),
+        ("smem_per_block", C.c_int64), ("smem_per_sm", C.c_int64),
+        ("smem_per_block_optin", C.c_int64),
+        ("mem_bandwidth_gb", C.c_double), ("base_clock_mhz", C.c_double),
+        ("peak_gflops", C.c_double),
+    ]
+
+
+class HabitatLibraryError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        super().__init__("%s failed: %s (code %d)" % (what, strerror(code), code))
+
+
+_lib = None
+
+_P = C.c_void_p
+_SIGNATURES = {
+    "hbt_version": (C.c_int, []),
+    "hbt_strerror": (C.c_char_p, [C.c_int]),
+    "hbt_device_count": (C.c_int, []),
+    "hbt_device_spec_check": (C.c_int, [C.POINTER(DeviceSpec)]),
+    "hbt_occupancy_host": (C.c_int, [C.POINTER(DeviceSpec), C.c_int32, C.c_int32, C.c_int32,
+                                     C.c_int32, C.POINTER(C.c_uint32)]),
+    "hbt_occupancy_host_batch": (C.c_int, [C.POINTER(DeviceSpec), C.c_int64, _P, _P, _P, _P, _P]),
+    "hbt_wave_scale": (C.c_int, [C.POINTER(DeviceSpec), C.POINTER(DeviceSpec), C.c_int32,
+                                 C.c_int64] + [_P] * 17 + [_P]),
+    "hbt_mlp_create": (_P, [C.c_int32, C.c_int32, C.c_int32, C.POINTER(_P), C.POINTER(_P), _P, _P,
+                            C.POINTER(C.c_int)]),
+    "hbt_mlp_forward": (C.c_int, [_P, _P, C.c_int64, _P, _P]),
+    "hbt_mlp_destroy": (None, [_P]),
+}
+
+# Entry points added after the first release of the ABI; bound when present.
+_OPTIONAL = {}
+
+
+def exported_symbols():
+    """Names include/habitat_mi.h declares."""
+    return sorted(list(_SIGNATURES) + list(_OPTIONAL))
+
+
+def lib():
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                "habitat_amd: %s is missing — build it with `python -m habitat_amd.build` "
+                "(there is no CPU fallback)" % LIB_PATH)
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in list(_SIGNATURES.items()) + list(_OPTIONAL.items()):
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def strerror(code):
+    return lib().hbt_strerror(code).decode()
+
+
+def check(code, what):
+    if code != HBT_OK:
+        raise HabitatLibraryError(code, what)

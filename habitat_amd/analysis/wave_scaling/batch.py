@@ -1,0 +1,126 @@
+"""Batched wave scaling: structure-of-arrays kernel records in HBM, one HIP
+launch per (origin, up to 8 destinations).
+
+This is the entry the scalar strategies (roofline.py, resimplified.py,
+unified.py in this package) are thin wrappers of.  It stands in for the
+reference's per-kernel loop (analyzer/habitat/analysis/predictor.py:116-124).
+torch is used only to own device memory and to name the stream.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from habitat_amd import _lib
+
+INT_COLUMNS = ("num_blocks", "block_size", "dynamic_smem", "static_smem", "regs_per_thread")
+F64_COLUMNS = ("run_time_ns", "flop_sp_efficiency", "dram_read_bytes", "dram_write_bytes")
+
+
+class KernelRecords:
+    """Kernel records as columns on one GPU.
+
+    Columns (length n): the launch geometry and resource use of
+    cpp/src/cuda/kernel.h:64-151 as int32 (`num_blocks` = grid x*y*z), the
+    measured time and the three metrics of wave_scaling/roofline.py:69-71 as
+    float64.  Optional: `dest_regs` (int32, < 0 = no entry in the register
+    table for the destination architecture) and `has_metrics` (uint8).
+    """
+
+    def __init__(self, columns, dest_regs=None, has_metrics=None):
+        n = None
+        self.columns = {}
+        for name in INT_COLUMNS + F64_COLUMNS:
+            t = columns[name]
+            want = torch.int32 if name in INT_COLUMNS else torch.float64
+            if not isinstance(t, torch.Tensor) or t.dtype != want or t.dim() != 1:
+                raise TypeError("column %s must be a 1-D %s tensor" % (name, want))
+            if not t.is_cuda:
+                raise ValueError("column %s must live on the GPU" % name)
+            t = t.contiguous()
+            n = t.shape[0] if n is None else n
+            if t.shape[0] != n:
+                raise ValueError("column %s has length %d, expected %d" % (name, t.shape[0], n))
+            self.columns[name] = t
+        self.n = int(n)
+        self.device = self.columns["num_blocks"].device
+        self.dest_regs = self._optional(dest_regs, torch.int32, "dest_regs")
+        self.has_metrics = self._optional(has_metrics, torch.uint8, "has_metrics")
+
+    def _optional(self, t, dtype, name):
+        if t is None:
+            return None
+        if t.dtype != dtype or t.dim() != 1 or t.shape[0] != self.n or not t.is_cuda:
+            raise TypeError("%s must be a 1-D %s GPU tensor of length %d" % (name, dtype, self.n))
+        return t.contiguous()
+
+    def __len__(self):
+        return self.n
+
+    @classmethod
+    def from_numpy(cls, rec, device="cuda"):
+        """Upload a dict of numpy columns (synchronous copy)."""
+        cols = {}
+        for name in INT_COLUMNS:
+            cols[name] = torch.from_numpy(np.ascontiguousarray(rec[name], np.int32)).to(device)
+        for name in F64_COLUMNS:
+            cols[name] = torch.from_numpy(np.ascontiguousarray(rec[name], np.float64)).to(device)
+        dr = rec.get("dest_regs")
+        hm = rec.get("has_metrics")
+        if dr is not None:
+            dr = torch.from_numpy(np.ascontiguousarray(dr, np.int32)).to(device)
+        if hm is not None:
+            hm = torch.from_numpy(np.ascontiguousarray(hm, np.uint8)).to(device)
+        return cls(cols, dr, hm)
+
+
+class WaveScaleOutput:
+    """Preallocated outputs of one `wave_scale` call (all on the GPU).
+
+    time_ns, occ_dest, wave_dest, status: [n_dest, n]; occ_origin, wave_origin: [n].
+    """
+
+    def __init__(self, n, n_dest, device, waves=True, status=True):
+        self.n, self.n_dest = n, n_dest
+        self.time_ns = torch.empty((n_dest, n), dtype=torch.float64, device=device)
+        self.occ_origin = torch.empty((n,), dtype=torch.int32, device=device)
+        self.occ_dest = torch.empty((n_dest, n), dtype=torch.int32, device=device)
+        self.wave_origin = torch.empty((n,), dtype=torch.int32, device=device) if waves else None
+        self.wave_dest = (torch.empty((n_dest, n), dtype=torch.int32, device=device)
+                          if waves else None)
+        self.status = torch.empty((n_dest, n), dtype=torch.uint8, device=device) if status else None
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def wave_scale(records, origin, dests, out=None, stream=None, waves=True, status=True):
+    """Scale every record from `origin` to each device in `dests`.
+
+    `origin` and the items of `dests` are DeviceProperties.  Returns a
+    WaveScaleOutput (the one passed in `out`, if any); the work is enqueued on
+    `stream` (default: torch's current stream) and not synchronised.
+    """
+    if not isinstance(dests, (list, tuple)):
+        dests = [dests]
+    n_dest = len(dests)
+    if out is None:
+        out = WaveScaleOutput(records.n, n_dest, records.device, waves=waves, status=status)
+    elif out.n != records.n or out.n_dest != n_dest:
+        raise ValueError("output buffers were allocated for another shape")
+    specs = (_lib.DeviceSpec * max(n_dest, 1))(*[d.spec for d in dests])
+    if stream is None:
+        stream = torch.cuda.current_stream(records.device)
+    c = records.columns
+    with torch.cuda.device(records.device):
+        rc = _lib.lib().hbt_wave_scale(
+            ctypes.byref(origin.spec), specs, n_dest, records.n,
+            _ptr(c["num_blocks"]), _ptr(c["block_size"]), _ptr(c["dynamic_smem"]),
+            _ptr(c["static_smem"]), _ptr(c["regs_per_thread"]), _ptr(records.dest_regs),
+            _ptr(c["run_time_ns"]), _ptr(c["flop_sp_efficiency"]), _ptr(c["dram_read_bytes"]),
+            _ptr(c["dram_write_bytes"]), _ptr(records.has_metrics),
+            _ptr(out.time_ns), _ptr(out.occ_origin), _ptr(out.occ_dest), _ptr(out.wave_origin),
+            _ptr(out.wave_dest), _ptr(out.status), ctypes.c_void_p(stream.cuda_stream))
+    _lib.check(rc, "hbt_wave_scale")
+    return out

@@ -1,0 +1,392 @@
+// Per-operation MLP inference on gfx950: the whole network in one kernel.
+//
+// Network (analyzer/habitat/analysis/mlp/mlp.py:17-109): fc1 (F -> W), ReLU,
+// `hidden` x [Linear(W, W), ReLU], fc2 (W -> 1), with W = 1024.  Input rows are
+// standardised as RuntimePredictor.predict does (mlp.py:258-264): (x - mu) /
+// sigma in fp64, then cast to fp32.
+//
+// Design.  A workgroup owns 32 input rows for the whole chain.  Their
+// activations (32 x 1024 fp32 = 128 KiB) live in LDS and never touch HBM; the
+// only global traffic in steady state is the weight stream, which every
+// workgroup reads in the same order and therefore mostly finds in L2.  A layer
+// is computed transposed, Out^T[n][m] = sum_k W[n][k] * Act[m][k], with
+// v_mfma_f32_32x32x2_f32: the A operand is a 32(n) x 2(k) weight fragment, the
+// B operand a 2(k) x 32(m) activation fragment.  The 32 n-tiles of a layer are
+// split over the waves; a wave keeps its slice of the output in accumulator
+// registers for the whole K loop and only then, after a barrier, overwrites the
+// LDS activations in place (bias enters as the accumulator's initial value,
+// ReLU is applied on the way out).
+//
+// Weights are repacked once, at hbt_mlp_create, so that a wave's fragment for
+// 8 consecutive k is one fully coalesced 1 KiB load (16 B per lane) straight
+// into the registers the MFMA reads: index [wave][k/8][tile][lane][4] holds
+// W[32*tile_global + lane%32][8*(k/8) + 4*(lane/32) + e].  The matching
+// activation fragment is one ds_read_b128 of Act[lane%32][8*(k/8) + 4*(lane/32) ..+3];
+// rows are padded by 4 floats so those reads are bank-conflict free.
+//
+// FLOPs per row: 2 * (F*1024 + hidden*1024^2 + 1024); bound: fp32 MFMA rate.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "../../include/habitat_mi.h"
+
+namespace hbt {
+
+namespace {
+
+using f32x4 = float __attribute__((ext_vector_type(4)));
+using f32x16 = float __attribute__((ext_vector_type(16)));
+
+constexpr int kWidth = 1024;      // hidden width the kernel is built for
+constexpr int kRows = 32;         // rows per workgroup (one MFMA tile of m)
+constexpr int kStride = kWidth + 4;  // LDS row stride in floats
+constexpr int kMaxInPadded = 64;  // in_features padded to a multiple of 16, at most this
+
+struct MlpArgs {
+  const double* raw;     // [n][in_features]
+  float* out;            // [n]
+  int64_t n;
+  int32_t in_features;
+  int32_t in_padded;     // multiple of 16
+  int32_t hidden;
+  const double* mu;      // [in_features]
+  const double* sigma;   // [in_features]
+  const float* w_first;  // packed fc1 [waves][in_padded/8][tpw][64][4]
+  const float* w_hidden; // packed hidden layers, kWidth*kWidth floats each
+  const float* bias;     // [(hidden + 1)][kWidth]: fc1 bias, then hidden biases
+  const float* w_last;   // fc2.weight [kWidth]
+  float b_last;
+};
+
+// One layer's K loop for this wave: acc[tile] += Wfrag * Actfrag over kg groups of 8 k.
+template <int TPW>
+__device__ __forceinline__ void layer_k_loop(const f32x4* __restrict__ wp, int kg,
+                                             const float* act_lane, f32x16 (&acc)[TPW]) {
+  const int lane = threadIdx.x & 63;
+  f32x4 wa[TPW], wb[TPW];
+  f32x4 xa, xb;
+#pragma unroll
+  for (int t = 0; t < TPW; ++t) wa[t] = wp[t * 64 + lane];
+  xa = *reinterpret_cast<const f32x4*>(act_lane);
+  for (int j = 0; j < kg; j += 2) {
+    // The scheduling barriers keep the compiler from sinking the prefetches
+    // below the MFMA block they are meant to overlap with.
+    {
+      const f32x4* p = wp + (size_t)(j + 1) * TPW * 64 + lane;
+#pragma unroll
+      for (int t = 0; t < TPW; ++t) wb[t] = p[t * 64];
+      xb = *reinterpret_cast<const f32x4*>(act_lane + 8 * (j + 1));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int t = 0; t < TPW; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[t][e], xa[e], acc[t], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      const int jn = (j + 2 < kg) ? (j + 2) : j;  // last iteration reloads a valid group
+      const f32x4* p = wp + (size_t)jn * TPW * 64 + lane;
+#pragma unroll
+      for (int t = 0; t < TPW; ++t) wa[t] = p[t * 64];
+      xa = *reinterpret_cast<const f32x4*>(act_lane + 8 * jn);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int t = 0; t < TPW; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(wb[t][e], xb[e], acc[t], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs a) {
+  constexpr int TPW = (kWidth / 32) / WAVES;  // n-tiles per wave
+  constexpr int THREADS = WAVES * 64;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* act = lds;                           // [kRows][kStride]
+  float* red = lds + kRows * kStride;         // [THREADS / 32][32]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 31, h = lane >> 5;
+  const int64_t row0 = (int64_t)blockIdx.x * kRows;
+
+  // ---- stage standardised inputs: act[r][k], zero beyond in_features / n ----
+  for (int idx = tid; idx < kRows * a.in_padded; idx += THREADS) {
+    const int r = idx / a.in_padded, k = idx - r * a.in_padded;
+    float v = 0.f;
+    if (k < a.in_features && row0 + r < a.n) {
+      const double x = a.raw[(row0 + r) * a.in_features + k];
+      v = (float)((x - a.mu[k]) / a.sigma[k]);
+    }
+    act[r * kStride + k] = v;
+  }
+  __syncthreads();
+
+  const float* act_lane = act + m * kStride + 4 * h;
+  const int tile0 = wave * TPW;  // first n-tile of this wave
+
+  f32x16 acc[TPW];
+  for (int layer = 0; layer <= a.hidden; ++layer) {
+    // accumulators start at the bias of their output column
+    const float* bias = a.bias + (size_t)layer * kWidth;
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 b = *reinterpret_cast<const f32x4*>(bias + (tile0 + t) * 32 + 8 * g + 4 * h);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[t][4 * g + e] = b[e];
+      }
+
+    if (layer == 0) {
+      const int kg = a.in_padded / 8;
+      const f32x4* wp = reinterpret_cast<const f32x4*>(a.w_first) + (size_t)wave * kg * TPW * 64;
+      layer_k_loop<TPW>(wp, kg, act_lane, acc);
+    } else {
+      constexpr int kg = kWidth / 8;
+      const f32x4* wp = reinterpret_cast<const f32x4*>(a.w_hidden) +
+                        ((size_t)(layer - 1) * WAVES + wave) * kg * TPW * 64;
+      layer_k_loop<TPW>(wp, kg, act_lane, acc);
+    }
+
+    __syncthreads();  // every wave has finished reading this layer's input
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = fmaxf(acc[t][4 * g + e], 0.f);
+        *reinterpret_cast<f32x4*>(act + m * kStride + (tile0 + t) * 32 + 8 * g + 4 * h) = o;
+      }
+    __syncthreads();
+  }
+
+  // ---- fc2: out[r] = sum_n act[r][n] * w_last[n] + b_last ----
+  {
+    constexpr int PARTS = THREADS / 32;
+    constexpr int NPP = kWidth / PARTS;
+    const int r = tid & 31, part = tid >> 5;
+    const float* ap = act + r * kStride + part * NPP;
+    const float* wl = a.w_last + part * NPP;
+    float s = 0.f;
+#pragma unroll 8
+    for (int k = 0; k < NPP; k += 4) {
+      const f32x4 x = *reinterpret_cast<const f32x4*>(ap + k);
+      const f32x4 w = *reinterpret_cast<const f32x4*>(wl + k);
+      s = fmaf(x[0], w[0], s);
+      s = fmaf(x[1], w[1], s);
+      s = fmaf(x[2], w[2], s);
+      s = fmaf(x[3], w[3], s);
+    }
+    red[part * 32 + r] = s;
+    __syncthreads();
+    if (tid < 32 && row0 + tid < a.n) {
+      float total = a.b_last;
+#pragma unroll
+      for (int p = 0; p < PARTS; ++p) total += red[p * 32 + tid];
+      a.out[row0 + tid] = total;
+    }
+  }
+}
+
+constexpr int kWaves = 8;
+constexpr size_t kLdsBytes = (size_t)(kRows * kStride + (kWaves * 64 / 32) * 32) * sizeof(float);
+
+}  // namespace
+
+}  // namespace hbt
+
+struct hbt_mlp {
+  int32_t in_features, in_padded, width, hidden;
+  int device;
+  void* blob;          // one device allocation holding everything below
+  const double* mu;
+  const double* sigma;
+  const float* w_first;
+  const float* w_hidden;
+  const float* bias;
+  const float* w_last;
+  float b_last;
+};
+
+namespace hbt {
+namespace {
+
+// Repack a row-major [kWidth][k_in] weight matrix (k_in <= k_padded) into
+// [waves][k_padded/8][tpw][64 lanes][4].
+void pack_layer(const float* W, int k_in, int k_padded, int waves, float* dst) {
+  const int tpw = (kWidth / 32) / waves;
+  const int kg = k_padded / 8;
+  for (int w = 0; w < waves; ++w)
+    for (int j = 0; j < kg; ++j)
+      for (int t = 0; t < tpw; ++t)
+        for (int lane = 0; lane < 64; ++lane)
+          for (int e = 0; e < 4; ++e) {
+            const int n = (w * tpw + t) * 32 + (lane & 31);
+            const int k = 8 * j + 4 * (lane >> 5) + e;
+            const float v = (k < k_in) ? W[(size_t)n * k_in + k] : 0.f;
+            dst[((((size_t)w * kg + j) * tpw + t) * 64 + lane) * 4 + e] = v;
+          }
+}
+
+size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+}  // namespace
+}  // namespace hbt
+
+extern "C" {
+
+hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layers,
+                        const float* const* W, const float* const* b, const double* mu,
+                        const double* sigma, int* err) {
+  using namespace hbt;
+  int dummy;
+  if (err == nullptr) err = &dummy;
+  *err = HBT_OK;
+  if (W == nullptr || b == nullptr || mu == nullptr || sigma == nullptr || in_features <= 0 ||
+      hidden_layers < 0) {
+    *err = HBT_EINVAL;
+    return nullptr;
+  }
+  for (int i = 0; i < hidden_layers + 2; ++i)
+    if (W[i] == nullptr || b[i] == nullptr) { *err = HBT_EINVAL; return nullptr; }
+  const int in_padded = (int)align_up((size_t)in_features, 16);
+  if (width != kWidth || in_padded > kMaxInPadded || hidden_layers > 64) {
+    *err = HBT_ESIZE;
+    return nullptr;
+  }
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    *err = HBT_EHIP;
+    return nullptr;
+  }
+
+  // Host image of the device blob.
+  const size_t n_first = (size_t)kWidth * in_padded;
+  const size_t n_hidden = (size_t)hidden_layers * kWidth * kWidth;
+  const size_t n_bias = (size_t)(hidden_layers + 1) * kWidth;
+  size_t off = 0;
+  const size_t off_mu = off; off = align_up(off + sizeof(double) * in_features, 256);
+  const size_t off_sigma = off; off = align_up(off + sizeof(double) * in_features, 256);
+  const size_t off_first = off; off = align_up(off + sizeof(float) * n_first, 256);
+  const size_t off_hidden = off; off = align_up(off + sizeof(float) * n_hidden, 256);
+  const size_t off_bias = off; off = align_up(off + sizeof(float) * n_bias, 256);
+  const size_t off_last = off; off = align_up(off + sizeof(float) * kWidth, 256);
+  const size_t total = off;
+
+  std::vector<unsigned char> host;
+  try {
+    host.resize(total, 0);
+  } catch (const std::bad_alloc&) {
+    *err = HBT_ENOMEM;
+    return nullptr;
+  }
+  std::memcpy(host.data() + off_mu, mu, sizeof(double) * in_features);
+  std::memcpy(host.data() + off_sigma, sigma, sizeof(double) * in_features);
+  pack_layer(W[0], in_features, in_padded, kWaves, reinterpret_cast<float*>(host.data() + off_first));
+  for (int l = 0; l < hidden_layers; ++l)
+    pack_layer(W[1 + l], kWidth, kWidth, kWaves,
+               reinterpret_cast<float*>(host.data() + off_hidden) + (size_t)l * kWidth * kWidth);
+  for (int l = 0; l <= hidden_layers; ++l)
+    std::memcpy(host.data() + off_bias + sizeof(float) * (size_t)l * kWidth, b[l],
+                sizeof(float) * kWidth);
+  std::memcpy(host.data() + off_last, W[hidden_layers + 1], sizeof(float) * kWidth);
+
+  void* blob = nullptr;
+  if (hipMalloc(&blob, total) != hipSuccess) {
+    (void)hipGetLastError();
+    *err = HBT_ENOMEM;
+    return nullptr;
+  }
+  if (hipMemcpy(blob, host.data(), total, hipMemcpyHostToDevice) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipFree(blob);
+    *err = HBT_EHIP;
+    return nullptr;
+  }
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&mlp_fused_kernel<kWaves>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (int)kLdsBytes) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipFree(blob);
+    *err = HBT_EHIP;
+    return nullptr;
+  }
+
+  hbt_mlp* m = new (std::nothrow) hbt_mlp();
+  if (m == nullptr) {
+    (void)hipFree(blob);
+    *err = HBT_ENOMEM;
+    return nullptr;
+  }
+  unsigned char* base = static_cast<unsigned char*>(blob);
+  m->in_features = in_features;
+  m->in_padded = in_padded;
+  m->width = width;
+  m->hidden = hidden_layers;
+  m->device = device;
+  m->blob = blob;
+  m->mu = reinterpret_cast<const double*>(base + off_mu);
+  m->sigma = reinterpret_cast<const double*>(base + off_sigma);
+  m->w_first = reinterpret_cast<const float*>(base + off_first);
+  m->w_hidden = reinterpret_cast<const float*>(base + off_hidden);
+  m->bias = reinterpret_cast<const float*>(base + off_bias);
+  m->w_last = reinterpret_cast<const float*>(base + off_last);
+  m->b_last = b[hidden_layers + 1][0];
+  return m;
+}
+
+int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* out,
+                    void* hip_stream) {
+  using namespace hbt;
+  if (mlp == nullptr || n < 0) return HBT_EINVAL;
+  if (n == 0) return HBT_OK;
+  if (raw_features == nullptr || out == nullptr) return HBT_EINVAL;
+  if ((reinterpret_cast<uintptr_t>(raw_features) % 8) != 0 ||
+      (reinterpret_cast<uintptr_t>(out) % 4) != 0)
+    return HBT_EALIGN;
+  const int64_t blocks = (n + kRows - 1) / kRows;
+  if (blocks > 0x7fffffff) return HBT_ESIZE;
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    return HBT_EHIP;
+  }
+  if (device != mlp->device) return HBT_EINVAL;
+
+  MlpArgs a{};
+  a.raw = raw_features;
+  a.out = out;
+  a.n = n;
+  a.in_features = mlp->in_features;
+  a.in_padded = mlp->in_padded;
+  a.hidden = mlp->hidden;
+  a.mu = mlp->mu;
+  a.sigma = mlp->sigma;
+  a.w_first = mlp->w_first;
+  a.w_hidden = mlp->w_hidden;
+  a.bias = mlp->bias;
+  a.w_last = mlp->w_last;
+  a.b_last = mlp->b_last;
+  hipLaunchKernelGGL(mlp_fused_kernel<kWaves>, dim3((unsigned)blocks), dim3(kWaves * 64),
+                     kLdsBytes, static_cast<hipStream_t>(hip_stream), a);
+  return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
+}
+
+void hbt_mlp_destroy(hbt_mlp* mlp) {
+  if (mlp == nullptr) return;
+  if (mlp->blob != nullptr) (void)hipFree(mlp->blob);
+  delete mlp;
+}
+
+}  // extern "C"

@@ -1,0 +1,62 @@
+// Kernel-argument block of the wave-scaling kernel and its launcher.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "occupancy.h"
+
+namespace hbt {
+
+// Destinations handled by one launch; more are processed in successive launches.
+constexpr int kMaxDestPerLaunch = 8;
+
+// Everything about one (origin, destination) pair that does not depend on the
+// record, computed in fp64 on the host in the reference's operation order
+// (analyzer/habitat/analysis/wave_scaling/roofline.py:48-64, :107-108).
+struct DestArgs {
+  OccDevice dev;
+  double sms;                  // num_sms as a double
+  double ridge;                // peak_gflops / mem_bandwidth_gb
+  double half_ridge;           // 0.5 * ridge
+  double neg_half_over_ridge;  // -0.5 / ridge
+  double bw_ratio;             // origin.mem_bandwidth_gb / dest.mem_bandwidth_gb
+  double clk_ratio;            // origin.base_clock_mhz / dest.base_clock_mhz
+  double log2_bw;              // log2(bw_ratio)
+  double log2_clk_sm;          // log2(clk_ratio) + log2(origin.num_sms / dest.num_sms)
+};
+
+struct WaveScaleArgs {
+  int64_t n;
+  int32_t n_dest;
+  int32_t write_origin;  // 1: this launch writes the per-record origin outputs
+  const int32_t* num_blocks;
+  const int32_t* block_size;
+  const int32_t* dynamic_smem;
+  const int32_t* static_smem;
+  const int32_t* regs;
+  const int32_t* dest_regs;    // nullable
+  const double* run_time_ns;
+  const double* flop_sp_efficiency;
+  const double* dram_read_bytes;
+  const double* dram_write_bytes;
+  const uint8_t* has_metrics;  // nullable
+  double* out_time_ns;         // [n_dest][n]
+  int32_t* out_occ_origin;     // [n], nullable
+  int32_t* out_occ_dest;       // [n_dest][n], nullable
+  int32_t* out_wave_origin;    // [n], nullable
+  int32_t* out_wave_dest;      // [n_dest][n], nullable
+  uint8_t* out_status;         // [n_dest][n], nullable
+  OccDevice origin;
+  double origin_peak_gflops;
+  double origin_sms;
+  DestArgs dest[kMaxDestPerLaunch];
+};
+
+DestArgs make_dest_args(const hbt_device_spec& origin, const hbt_device_spec& dest);
+
+// `vectorised` needs every column 16-byte aligned (and n % 4 == 0 when n_dest > 1).
+hipError_t launch_wave_scale(const WaveScaleArgs& args, bool vectorised, hipStream_t stream);
+
+}  // namespace hbt

@@ -1,0 +1,156 @@
+/*
+ * habitat_mi — C ABI of the MI355X-native batched-prediction path.
+ *
+ * This is the whole boundary between host code (Python via ctypes, or any
+ * other FFI) and the HIP kernels.  Plain pointers and sizes only.  Unless a
+ * parameter says "host", every array pointer is DEVICE memory owned by the
+ * caller; work is enqueued on the given HIP stream (NULL = the default stream)
+ * and the call returns without synchronising.  Functions return 0 or a
+ * negative HBT_E* code; hbt_strerror() names it.  There is no global state and
+ * no CPU fallback: without a GPU the compute entry points return HBT_EHIP.
+ *
+ * Each entry point cites the reference interface it stands in for
+ * (paths relative to the reference tree).
+ */
+#ifndef HABITAT_MI_H_
+#define HABITAT_MI_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HBT_VERSION 100 /* 0.1.0 */
+
+enum {
+  HBT_OK = 0,
+  HBT_EINVAL = -1, /* null pointer, negative count, bad argument */
+  HBT_ESPEC = -2,  /* device spec outside the supported domain (see hbt_device_spec_check) */
+  HBT_EHIP = -3,   /* a HIP runtime call failed (no GPU, bad stream, launch error) */
+  HBT_ENOMEM = -4, /* device allocation failed (hbt_mlp_create only) */
+  HBT_EALIGN = -5, /* a column pointer is not aligned to its element size */
+  HBT_ESIZE = -6   /* size beyond what the entry point supports */
+};
+
+/* Per-record status written by hbt_wave_scale.  Non-zero statuses are the
+ * places where the reference's scalar Python raises instead of returning; the
+ * predicted time of such a record is NaN. */
+enum {
+  HBT_ST_OK = 0,
+  HBT_ST_ORIGIN_WAVE_ZERO = 1, /* ZeroDivisionError at wave_scaling/roofline.py:29, resimplified.py:25 */
+  HBT_ST_DEST_WAVE_ZERO = 2,   /* ZeroDivisionError at wave_scaling/roofline.py:30, resimplified.py:26 */
+  HBT_ST_BAD_GAMMA = 3,        /* AssertionError at wave_scaling/roofline.py:103 */
+  HBT_ST_ZERO_BLOCKS = 4       /* ZeroDivisionError at wave_scaling/roofline.py:40 (num_blocks == 0) */
+};
+
+/*
+ * Device description.  Replaces habitat::cuda::DeviceProperties
+ * (cpp/src/cuda/kernel.h:14-62; Python constructor
+ * cpp/src/frontend/model_bindings.cpp:17-55) minus the name, which stays on
+ * the host side.  The three double fields hold integer values, as the
+ * reference's fields are integers (kernel.h:59-61).
+ */
+typedef struct hbt_device_spec {
+  int32_t compute_major, compute_minor;
+  int32_t max_threads_per_block, max_threads_per_sm;
+  int32_t regs_per_block, regs_per_sm;
+  int32_t warp_size, num_sms;
+  int64_t smem_per_block, smem_per_sm, smem_per_block_optin;
+  double mem_bandwidth_gb, base_clock_mhz, peak_gflops;
+} hbt_device_spec;
+
+int hbt_version(void);
+const char *hbt_strerror(int code);
+
+/* Number of HIP devices visible to the library (0 without a GPU); never fails. */
+int hbt_device_count(void);
+
+/*
+ * HBT_OK when `spec` (host) is inside the domain the batch kernels accept:
+ * smem fields >= 0 and < 2^31, warp_size <= 32768, num_sms <= 2^26,
+ * mem_bandwidth_gb, base_clock_mhz, peak_gflops finite and > 0.  A spec the
+ * occupancy model rejects (unknown compute capability, a zero limit) is still
+ * in the domain: every occupancy on it is 0, as in the reference.
+ */
+int hbt_device_spec_check(const hbt_device_spec *spec);
+
+/*
+ * Thread-block occupancy of one launch configuration on one device, on the
+ * HOST (all pointers host).  Replaces KernelMetadata::threadBlockOccupancy
+ * (cpp/src/cuda/kernel.h:104-115, cpp/src/cuda/kernel.cpp:29-56) and its Python
+ * face KernelInstance.thread_block_occupancy
+ * (cpp/src/frontend/model_bindings.cpp:75-82).  `regs` is narrowed to 16 bits
+ * as there; any error in the model gives *out = 0.
+ */
+int hbt_occupancy_host(const hbt_device_spec *spec, int32_t block_size, int32_t dynamic_smem,
+                       int32_t static_smem, int32_t regs, uint32_t *out);
+
+/* The same over host arrays (used by data generators and host-side callers). */
+int hbt_occupancy_host_batch(const hbt_device_spec *spec, int64_t n, const int32_t *block_size,
+                             const int32_t *dynamic_smem, const int32_t *static_smem,
+                             const int32_t *regs, int32_t *out);
+
+/*
+ * Wave-scale n kernel records measured on `origin` to each of n_dest
+ * destination devices.  One launch replaces the per-kernel Python loop of
+ * Predictor._wave_scale (analyzer/habitat/analysis/predictor.py:116-124) and,
+ * per record, unified_wave_scaling (analysis/wave_scaling/unified.py:8-35) with
+ * everything under it: roofline.py:8-108, resimplified.py:7-40,
+ * common.py:3-20 and the occupancy routine above.
+ *
+ * origin, dests: HOST pointers (dests is an array of n_dest specs).
+ * Input columns (device, length n): the fields of KernelMetadata /
+ * KernelInstance (cpp/src/cuda/kernel.h:64-151) and the three metrics that
+ * roofline.py:69-71 reads.
+ *   dest_regs    nullable; >= 0 replaces regs for the destination occupancy
+ *                (MetadataManager.kernel_registers_for, wave_scaling/metadata.py:12-37;
+ *                < 0 = no entry)
+ *   has_metrics  nullable (= all present); 0 selects the no-metrics strategy
+ * Outputs (device): out_time_ns, out_occ_dest, out_wave_dest, out_status are
+ * [n_dest][n] row-major; out_occ_origin, out_wave_origin are [n].
+ * out_wave_*, out_status and out_occ_* are nullable.
+ */
+int hbt_wave_scale(const hbt_device_spec *origin, const hbt_device_spec *dests, int32_t n_dest,
+                   int64_t n, const int32_t *num_blocks, const int32_t *block_size,
+                   const int32_t *dynamic_smem, const int32_t *static_smem, const int32_t *regs,
+                   const int32_t *dest_regs, const double *run_time_ns,
+                   const double *flop_sp_efficiency, const double *dram_read_bytes,
+                   const double *dram_write_bytes, const uint8_t *has_metrics,
+                   double *out_time_ns, int32_t *out_occ_origin, int32_t *out_occ_dest,
+                   int32_t *out_wave_origin, int32_t *out_wave_dest, uint8_t *out_status,
+                   void *hip_stream);
+
+/*
+ * Per-operation MLP (fc1 -> ReLU -> hidden x (Linear, ReLU) -> fc2), the
+ * network of analysis/mlp/mlp.py:17-109.  hbt_mlp_create takes HOST pointers:
+ * W[0] is fc1.weight [width][in_features], W[1..hidden] are the hidden
+ * weights [width][width], W[hidden+1] is fc2.weight [1][width], all row-major
+ * fp32 as in a torch state_dict; b[] likewise; mu and sigma are the
+ * checkpoint's normalisation vectors [in_features] (mlp.py:133-137).  The
+ * weights are copied to the current HIP device in the layout the kernels want;
+ * this is the only call that allocates.  Returns NULL on failure (and sets
+ * *err if err is not NULL).
+ */
+typedef struct hbt_mlp hbt_mlp;
+hbt_mlp *hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layers,
+                        const float *const *W, const float *const *b, const double *mu,
+                        const double *sigma, int *err);
+
+/*
+ * Batched RuntimePredictor.predict (analysis/mlp/mlp.py:252-267): rows of raw
+ * (un-normalised) features [n][in_features] fp64 — operation features then the
+ * four device features — are standardised in fp64, cast to fp32, and run
+ * through the network; out[n] receives the fp32 predictions.  Needs no
+ * workspace: activations stay on-chip between layers.  Must be called with
+ * the device of hbt_mlp_create current.
+ */
+int hbt_mlp_forward(hbt_mlp *mlp, const double *raw_features, int64_t n, float *out,
+                    void *hip_stream);
+void hbt_mlp_destroy(hbt_mlp *mlp);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HABITAT_MI_H_ */
