@@ -1,0 +1,235 @@
+#!/usr/bin/env python3
+"""Benchmark of the batched-prediction hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of wave scaling over the 1 M synthetic kernel records of
+BASELINE.json's configs[1] (V100-like origin -> MI355X-like destination),
+inputs resident in HBM.  Prints ONE JSON line:
+  value         whole-job wave-scaled kernel records per second (K steps, wall clock)
+  roofline      the wave-scaling kernel against HBM bandwidth: 68 algorithmic
+                bytes per record / average launch duration (HIP events on the
+                launch stream)
+  cpu_baseline  the CPU oracle (C restatement of the reference's per-kernel
+                Python, one thread) on the same records, same machine
+  large         the same kernel at 64 M records (beyond the 256 MB last-level cache)
+  mlp           the fused MFMA MLP (configs[2], conv2d, 1 M rows): rows/s, its
+                roofline against fp32 MFMA peak and a torch-CPU fp32 baseline
+Only one GPU is used; --gpus above 1 exits.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
+BYTES_PER_RECORD = 68          # 5 x i32 + 4 x f64 read, f64 + 2 x i32 written
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--records", type=int, default=1_000_000)
+    ap.add_argument("--large-records", type=int, default=64_000_000)
+    ap.add_argument("--mlp-rows", type=int, default=1_000_000)
+    ap.add_argument("--mlp-kind", default="conv2d")
+    ap.add_argument("--mlp-steps", type=int, default=3)
+    ap.add_argument("--no-mlp", action="store_true")
+    ap.add_argument("--no-large", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    return ap.parse_args()
+
+
+class WaveScaleCall:
+    """The C-ABI call with every argument converted once, so the timed loop
+    measures the library and the GPU rather than Python argument handling."""
+
+    def __init__(self, records, origin, dest, out):
+        import torch
+        from habitat_amd import _lib
+        self.lib = _lib.lib()
+        self.keep = (records, out, origin, dest)
+        p = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+        c = records.columns
+        self.stream = torch.cuda.current_stream()
+        self.args = (
+            ctypes.byref(origin.spec), ctypes.byref(dest.spec), 1, records.n,
+            p(c["num_blocks"]), p(c["block_size"]), p(c["dynamic_smem"]), p(c["static_smem"]),
+            p(c["regs_per_thread"]), p(records.dest_regs), p(c["run_time_ns"]),
+            p(c["flop_sp_efficiency"]), p(c["dram_read_bytes"]), p(c["dram_write_bytes"]),
+            p(records.has_metrics), p(out.time_ns), p(out.occ_origin), p(out.occ_dest),
+            p(out.wave_origin), p(out.wave_dest), p(out.status),
+            ctypes.c_void_p(self.stream.cuda_stream))
+
+    def __call__(self):
+        rc = self.lib.hbt_wave_scale(*self.args)
+        if rc != 0:
+            raise RuntimeError("hbt_wave_scale failed: %d" % rc)
+
+
+def time_steps(call, steps, warmup):
+    """(wall ms per step, event ms per launch) over exactly `steps` calls."""
+    import torch
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        call()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return wall_ms, e0.elapsed_time(e1) / steps
+
+
+def tile_records(rec, n):
+    import numpy as np
+    base = rec["num_blocks"].shape[0]
+    reps = (n + base - 1) // base
+    return {k: np.tile(v, reps)[:n] for k, v in rec.items()}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported "
+              "(records and rows are independent and would shard by ranges, see DESIGN.md)"
+              % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from habitat_amd import Device, synthetic
+    from habitat_amd.analysis.mlp.mlp import RuntimePredictor
+    from habitat_amd.analysis.wave_scaling.batch import KernelRecords, WaveScaleOutput
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    origin, dest = Device.V100, Device.MI355X
+
+    # ---------------- wave scaling, configs[1] ----------------
+    rec, stats = synthetic.kernel_records(args.records, origin, seed=0)
+    records = KernelRecords.from_numpy(rec)
+    out = WaveScaleOutput(records.n, 1, records.device, waves=False, status=True)
+    call = WaveScaleCall(records, origin, dest, out)
+    wall_ms, launch_ms = time_steps(call, args.steps, args.warmup)
+    rec_per_s = args.records / (wall_ms * 1e-3)
+    achieved = BYTES_PER_RECORD * args.records / (launch_ms * 1e-3) / 1e9
+    result = {
+        "metric": "wave-scaled kernel records/s (1 GPU); MLP op-predictions/s under 'mlp'",
+        "value": rec_per_s, "unit": "records/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": wall_ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": {"workload": "configs[1]: wave scaling, %d kernel records (SoA, int32 launch "
+                               "params, fp64 times/metrics), V100 -> MI355X-like, outputs time + "
+                               "2 occupancies + status" % args.records,
+                   "records": args.records, "origin": origin.name, "dest": dest.name,
+                   "seed": stats["seed"], "rejected_draws": stats["rejected"]},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "wave_scale_kernel<4>", "launch_us": launch_ms * 1e3,
+                     "bytes_per_record": BYTES_PER_RECORD},
+    }
+
+    # ---------------- CPU baseline on the same records ----------------
+    if not args.no_cpu:
+        from oracle import lib as olib
+        from oracle import wave_scaling as ows
+        o = olib.make_device(**origin.as_dict())
+        d = olib.make_device(**dest.as_dict())
+        olib.wave_scale(o, d, rec)
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t0 < 5.0 and reps < 100):
+            olib.wave_scale(o, d, rec)
+            reps += 1
+        c_rate = reps * args.records / (time.perf_counter() - t0)
+        m = min(100_000, args.records)
+        rows = [{k: v[i].item() for k, v in rec.items()} for i in range(m)]
+        t0 = time.perf_counter()
+        for row in rows:
+            ows.unified(row, o, d)
+        py_rate = m / (time.perf_counter() - t0)
+        result["cpu_baseline"] = {
+            "value": c_rate, "unit": "records/s", "cores": 1, "kind": "port",
+            "sample": "oracle/wave_scaling.c (per-record C restatement of the reference's "
+                      "Python, libm pow) over the same %d records x %d passes, one thread of %d "
+                      "host cores" % (args.records, reps, os.cpu_count()),
+            "python_per_record": {
+                "value": py_rate, "unit": "records/s", "cores": 1,
+                "sample": "oracle/wave_scaling.py, one Python call chain per record as the "
+                          "reference does, first %d records" % m}}
+
+    # ---------------- the same kernel beyond the last-level cache ----------------
+    if not args.no_large and args.large_records > args.records:
+        del call, records, out
+        big = KernelRecords.from_numpy(tile_records(rec, args.large_records))
+        big_out = WaveScaleOutput(big.n, 1, big.device, waves=False, status=True)
+        big_call = WaveScaleCall(big, origin, dest, big_out)
+        steps = max(5, min(args.steps, 30))
+        b_wall, b_launch = time_steps(big_call, steps, 3)
+        b_ach = BYTES_PER_RECORD * big.n / (b_launch * 1e-3) / 1e9
+        result["large"] = {"records": big.n, "steps": steps, "ms_per_step": b_wall,
+                           "value": big.n / (b_wall * 1e-3), "unit": "records/s",
+                           "roofline": {"bound": "hbm", "achieved": b_ach, "peak": HBM_PEAK_GBS,
+                                        "unit": "GB/s", "frac": b_ach / HBM_PEAK_GBS,
+                                        "launch_us": b_launch * 1e3}}
+        del big_call, big, big_out
+        torch.cuda.empty_cache()
+
+    # ---------------- MLP, configs[2] ----------------
+    if not args.no_mlp:
+        kind = args.mlp_kind
+        torch.manual_seed(0)
+        rp = RuntimePredictor(kind, 8, 1024)
+        x, mu, sigma = synthetic.mlp_features(kind, args.mlp_rows, seed=2)
+        rp.set_normalization(mu, sigma)
+        xg = torch.from_numpy(x).cuda()
+        yg = torch.empty(args.mlp_rows, dtype=torch.float32, device="cuda")
+        f_in = x.shape[1]
+        flops_per_row = 2.0 * (f_in * 1024 + 8 * 1024 * 1024 + 1024)
+        mlp_call = lambda: rp.predict_batch(xg, out=yg)
+        m_wall, m_launch = time_steps(mlp_call, args.mlp_steps, 1)
+        tflops = flops_per_row * args.mlp_rows / (m_launch * 1e-3) / 1e12
+        mlp = {"metric": "MLP op-predictions/s", "value": args.mlp_rows / (m_wall * 1e-3),
+               "unit": "rows/s", "steps": args.mlp_steps, "ms_per_step": m_wall, "dtype": "f32",
+               "config": {"workload": "configs[2]: %s MLP, %d rows x %d raw fp64 features, "
+                                      "fc1 + 8 x 1024 hidden + fc2, seed-0 random init"
+                                      % (kind, args.mlp_rows, f_in)},
+               "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_FP32_PEAK_TFLOPS,
+                            "unit": "TFLOP/s", "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
+                            "traffic": None, "kernel": "mlp_fused_kernel",
+                            "launch_ms": m_launch, "flops_per_row": flops_per_row}}
+        if not args.no_cpu:
+            from oracle import mlp as omlp
+            sd = rp.model.state_dict()
+            m = min(32768, args.mlp_rows)
+            threads = torch.get_num_threads()
+            omlp.forward_fp32(sd, x[:1024], mu, sigma)
+            t0 = time.perf_counter()
+            omlp.forward_fp32(sd, x[:m], mu, sigma)
+            dt = time.perf_counter() - t0
+            mlp["cpu_baseline"] = {
+                "value": m / dt, "unit": "rows/s", "cores": threads, "kind": "port",
+                "sample": "oracle/mlp.py forward_fp32 (torch CPU fp32, one batched forward) on "
+                          "the first %d rows, %d torch threads" % (m, threads)}
+        result["mlp"] = mlp
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,100 @@
+"""Kernel objects of the data model.
+
+`KernelInstance` is the record a profiler produces for one kernel launch: the
+Python face of the reference's C++ class (cpp/src/cuda/kernel.h:64-151,
+bindings cpp/src/frontend/model_bindings.cpp:57-82).  `MeasuredKernel` and
+`PredictedKernel` follow analyzer/habitat/analysis/kernels.py:3-44.
+"""
+
+
+class KernelInstance:
+    def __init__(self, name, num_blocks, block_size, dynamic_shared_memory,
+                 static_shared_memory, registers_per_thread, run_time_ns, metrics=None):
+        self._name = name
+        self._num_blocks = int(num_blocks)
+        self._block_size = int(block_size)
+        self._dynamic_shared_memory = int(dynamic_shared_memory)
+        self._static_shared_memory = int(static_shared_memory)
+        self._registers_per_thread = int(registers_per_thread) & 0xFFFF  # uint16_t
+        self._run_time_ns = int(run_time_ns)
+        self._metrics = list(metrics) if metrics is not None else []
+
+    @property
+    def name(self):
+        return self._name
+
+    @property
+    def run_time_ns(self):
+        return self._run_time_ns
+
+    @property
+    def num_blocks(self):
+        return self._num_blocks
+
+    @property
+    def metrics(self):
+        """[(raw metric name, value)]"""
+        return self._metrics
+
+    def add_metric(self, name, value):
+        self._metrics.append((name, float(value)))
+
+    @property
+    def metadata(self):
+        return {
+            "name": self._name,
+            "num_blocks": self._num_blocks,
+            "block_size": self._block_size,
+            "static_shared_memory": self._static_shared_memory,
+            "dynamic_shared_memory": self._dynamic_shared_memory,
+            "registers_per_thread": self._registers_per_thread,
+        }
+
+    def thread_block_occupancy(self, device, registers_per_thread=-1):
+        """Blocks per multiprocessor on `device`; a negative register count
+        means this kernel's own (model_bindings.cpp:75-82)."""
+        regs = self._registers_per_thread if registers_per_thread < 0 else registers_per_thread
+        return device.thread_block_occupancy(
+            self._block_size, self._dynamic_shared_memory, self._static_shared_memory, regs)
+
+
+class MeasuredKernel:
+    def __init__(self, time_kernel, metrics_kernels, device):
+        self._c = time_kernel
+        self._metrics_kernels = metrics_kernels
+        self._device = device
+        self._cached_metrics = {}
+
+    def get_metric(self, metric_info, default=None):
+        if metric_info in self._cached_metrics:
+            return self._cached_metrics[metric_info]
+        info = metric_info.value
+        for metric_kernel in self._metrics_kernels:
+            for raw_name, raw_value in metric_kernel.metrics:
+                if raw_name == info.cupti_name or raw_name == info.legacy_cupti_name:
+                    value = info.to_canonical_value(raw_value, self._device)
+                    self._cached_metrics[metric_info] = value
+                    return value
+        if default is None:
+            raise AttributeError("Unknown metric: {}".format(metric_info.name))
+        return default
+
+    def __getattr__(self, name):
+        # Everything else comes from the underlying kernel instance.
+        if name == "_c":
+            raise AttributeError(name)
+        return getattr(self._c, name)
+
+
+class PredictedKernel:
+    def __init__(self, measured_kernel, run_time_ns):
+        self._measured_kernel = measured_kernel
+        self._run_time_ns = run_time_ns
+
+    @property
+    def run_time_ns(self):
+        return self._run_time_ns
+
+    @property
+    def name(self):
+        return self._measured_kernel.name

@@ -1,0 +1,312 @@
+"""Routes each operation of a trace to wave scaling or to an MLP and assembles
+the predicted run times (analyzer/habitat/analysis/predictor.py:53-283).
+
+The reference predicts one kernel and one operation at a time.  Here
+`predict_operation` keeps that interface, while `predict_operations` and
+`predict_trace_times` gather every kernel record (resp. every MLP feature row)
+of a trace and hand them to the GPU in one call each.
+"""
+import functools
+import logging
+import operator
+import os
+
+import numpy as np
+import torch
+
+from habitat_amd.analysis import SPECIAL_OPERATIONS
+from habitat_amd.analysis.kernels import PredictedKernel
+from habitat_amd.analysis.metrics import Metric
+from habitat_amd.analysis.mlp.devices import get_device_features
+from habitat_amd.analysis.mlp.mlp import RuntimePredictor
+from habitat_amd.analysis.operation import PredictedOperation
+from habitat_amd.analysis.run_time import (RunTimePrediction, RunTimePurePrediction, ms_to_ns)
+from habitat_amd.analysis.wave_scaling.batch import KernelRecords, wave_scale
+from habitat_amd.analysis.wave_scaling.metadata import MetadataManager, NullMetadataManager
+from habitat_amd.analysis.wave_scaling.resimplified import resimplified_wave_scaling
+from habitat_amd.analysis.wave_scaling.roofline import roofline_wave_scaling
+from habitat_amd.analysis.wave_scaling.scalar import kernel_fields, raise_for_status
+from habitat_amd.analysis.wave_scaling.unified import unified_wave_scaling
+from habitat_amd.data import path_to_data
+
+logger = logging.getLogger(__name__)
+
+# Positional parameter names of the torch callables whose arguments were recorded.
+CONV2D_PARAMS = ["input", "weight", "bias", "stride", "padding", "dilation", "groups"]
+LINEAR_PARAMS = ["input", "weight", "bias"]
+BMM_PARAMS = ["input", "mat2", "out"]
+LSTM_PARAMS_NO_BATCH_SIZES = ["input", "hx", "flat_weights", "bias", "num_layers", "dropout",
+                              "training", "bidirectional", "batch_first"]
+LSTM_PARAMS = ["input", "batch_sizes", "hx", "flat_weights", "bias", "num_layers", "dropout",
+               "training", "bidirectional"]
+
+_METRICS = (Metric.SinglePrecisionFLOPEfficiency, Metric.DRAMReadBytes, Metric.DRAMWriteBytes)
+_MLP_KINDS = ("conv2d", "lstm", "linear", "bmm")
+
+
+def name_all_arguments(all_parameters, args, kwargs):
+    """Positional and keyword arguments merged under the declared parameter
+    names (analyzer/habitat/utils.py:54-63)."""
+    merged = dict(kwargs)
+    for arg_name, arg in zip(all_parameters, args):
+        merged[arg_name] = arg
+    return merged
+
+
+def _first(value):
+    return value[0] if isinstance(value, tuple) else value
+
+
+def conv2d_arguments(operation):
+    """predictor.py:150-173"""
+    m = name_all_arguments(CONV2D_PARAMS, operation.arguments.args, operation.arguments.kwargs)
+    return dict(batch=m["input"][0], image_size=m["input"][2], in_channels=m["input"][1],
+                out_channels=m["weight"][0], kernel_size=m["weight"][2],
+                stride=_first(m["stride"]), padding=_first(m["padding"]),
+                bias=(1 if m["bias"] is not None else 0))
+
+
+def linear_arguments(operation):
+    """predictor.py:184-211: the batch is the product of all leading dimensions."""
+    m = name_all_arguments(LINEAR_PARAMS, operation.arguments.args, operation.arguments.kwargs)
+    return dict(batch=functools.reduce(operator.mul, m["input"][:-1]),
+                in_features=m["weight"][1], out_features=m["weight"][0],
+                bias=(1 if m["bias"] is not None else 0))
+
+
+def bmm_arguments(operation):
+    """predictor.py:220-232"""
+    m = name_all_arguments(BMM_PARAMS, operation.arguments.args, operation.arguments.kwargs)
+    return dict(batch=m["input"][0], left=m["input"][1], middle=m["input"][2],
+                right=m["mat2"][2])
+
+
+def lstm_arguments(operation):
+    """predictor.py:240-276: the packed-sequence overload has a bool in position 4."""
+    args = operation.arguments.args
+    if not isinstance(args[4], bool):
+        m = name_all_arguments(LSTM_PARAMS_NO_BATCH_SIZES, args, operation.arguments.kwargs)
+        batch, seq_len, input_size = m["input"][1], m["input"][0], m["input"][2]
+    else:
+        m = name_all_arguments(LSTM_PARAMS, args, operation.arguments.kwargs)
+        batch = max(operation.arguments.special["batch_sizes"])
+        seq_len, input_size = m["input"][0] // batch, m["input"][1]
+    return dict(bias=(1 if m["bias"] is not None else 0),
+                bidirectional=(1 if m["bidirectional"] else 0), batch=batch, seq_len=seq_len,
+                input_size=input_size, hidden_size=m["hx"][0][2], num_layers=m["num_layers"])
+
+
+_ARGUMENTS = {"conv2d": conv2d_arguments, "linear": linear_arguments, "bmm": bmm_arguments,
+              "lstm": lstm_arguments}
+
+_BUILTIN = {unified_wave_scaling: "unified", roofline_wave_scaling: "roofline",
+            resimplified_wave_scaling: "resimplified"}
+
+
+def records_from_kernels(kernels, dest_device, metadata_manager, mode="unified", device=None):
+    """Python kernel objects -> KernelRecords on the GPU (one upload)."""
+    n = len(kernels)
+    ints = np.empty((5, n), np.int32)
+    f64 = np.zeros((4, n), np.float64)
+    has = np.zeros(n, np.uint8)
+    for i, k in enumerate(kernels):
+        nb, block, dyn, stat, regs, t_ns = kernel_fields(k)
+        ints[:, i] = (nb, block, dyn, stat, regs)
+        f64[0, i] = t_ns
+        if mode != "resimplified":
+            try:
+                f64[1:, i] = [k.get_metric(m) for m in _METRICS]
+                has[i] = 1
+            except AttributeError:
+                if mode == "roofline":
+                    raise
+    if hasattr(metadata_manager, "registers_for_names"):
+        dest_regs = metadata_manager.registers_for_names([k.name for k in kernels], dest_device)
+    else:
+        looked = [metadata_manager.kernel_registers_for(k, dest_device) for k in kernels]
+        dest_regs = [-1 if r is None else r for r in looked]
+    rec = {"num_blocks": ints[0], "block_size": ints[1], "dynamic_smem": ints[2],
+           "static_smem": ints[3], "regs_per_thread": ints[4], "run_time_ns": f64[0],
+           "flop_sp_efficiency": f64[1], "dram_read_bytes": f64[2], "dram_write_bytes": f64[3],
+           "dest_regs": np.asarray(dest_regs, np.int32), "has_metrics": has}
+    return KernelRecords.from_numpy(rec, device=device or "cuda")
+
+
+class Predictor:
+    def __init__(self, kernel_metadata_file=None, wave_scaling_strategy=unified_wave_scaling,
+                 mlp_predictors=None):
+        """`kernel_metadata_file`: sqlite register table (default: data/kernels.sqlite
+        if present, else no table).  `mlp_predictors`: {'conv2d'|'lstm'|'linear'|'bmm':
+        RuntimePredictor}; missing ones are loaded from data/<kind>/model.pth when
+        that file exists and are otherwise left without weights."""
+        default_lut = path_to_data("kernels.sqlite")
+        if kernel_metadata_file is not None:
+            self._kernel_metadata = MetadataManager(kernel_metadata_file)
+        elif os.path.exists(default_lut):
+            self._kernel_metadata = MetadataManager(default_lut)
+        else:
+            self._kernel_metadata = NullMetadataManager()
+        self._wave_scaling_strategy = wave_scaling_strategy
+
+        mlp_predictors = dict(mlp_predictors or {})
+        for kind in _MLP_KINDS:
+            if kind not in mlp_predictors:
+                path = path_to_data("%s/model.pth" % kind)
+                mlp_predictors[kind] = RuntimePredictor(
+                    kind, 8, 1024, path if os.path.exists(path) else None)
+        self.linear_pred = mlp_predictors["linear"]
+        self.lstm_pred = mlp_predictors["lstm"]
+        self.conv2d_pred = mlp_predictors["conv2d"]
+        self.bmm_pred = mlp_predictors["bmm"]
+
+    def _mlp(self, kind):
+        return getattr(self, kind + "_pred")
+
+    # ------------------------------------------------------------------ one op
+    def predict_operation(self, operation, dest_device):
+        return self.predict_operations([operation], dest_device)[0]
+
+    # ------------------------------------------------------------- many ops
+    def predict_operations(self, operations, dest_device):
+        """[PredictedOperation] for `operations`, with one wave-scaling launch
+        for all their kernels and one MLP launch per operation kind."""
+        results = [None] * len(operations)
+        scaled, special = [], {}
+        for i, op in enumerate(operations):
+            if op.name not in SPECIAL_OPERATIONS:
+                scaled.append(i)
+            elif op.name in _ARGUMENTS:
+                special.setdefault(op.name, []).append(i)
+            else:
+                logger.warning("Unhandled special operation: %s", op.name)
+                results[i] = PredictedOperation(op, op.forward, op.backward, dest_device)
+
+        if scaled:
+            passes = []  # (op index, is_backward, run_time)
+            for i in scaled:
+                op = operations[i]
+                passes.append((i, False, op.forward))
+                if op.backward is not None:
+                    passes.append((i, True, op.backward))
+            predicted = self._wave_scale_passes([p[2] for p in passes], dest_device)
+            fwd, bwd = {}, {}
+            for (i, is_bwd, _), pred in zip(passes, predicted):
+                (bwd if is_bwd else fwd)[i] = pred
+            for i in scaled:
+                results[i] = PredictedOperation(operations[i], fwd[i], bwd.get(i), dest_device)
+
+        for kind, idxs in special.items():
+            ops = [operations[i] for i in idxs]
+            for i, ms in zip(idxs, self._special_scale_many(kind, ops, dest_device)):
+                results[i] = PredictedOperation(
+                    operations[i], RunTimePurePrediction(ms, dest_device), None, dest_device)
+        return results
+
+    def _wave_scale(self, run_time, dest_device):
+        return self._wave_scale_passes([run_time], dest_device)[0]
+
+    def _wave_scale_passes(self, run_times, dest_device):
+        """predictor.py:111-130 for several passes at once."""
+        mode = _BUILTIN.get(self._wave_scaling_strategy)
+        out = []
+        if mode is None:
+            # A caller-supplied strategy: one call per kernel, as in the reference.
+            for rt in run_times:
+                preds = [self._wave_scaling_strategy(k, rt.device, dest_device,
+                                                     self._kernel_metadata) for k in rt.kernels]
+                out.append(self._assemble(rt, preds, dest_device))
+            return out
+
+        # Group passes by origin device; one launch per origin.
+        by_origin = {}
+        for idx, rt in enumerate(run_times):
+            by_origin.setdefault(rt.device.name, (rt.device, []))[1].append(idx)
+        times = [None] * len(run_times)
+        for origin, idxs in by_origin.values():
+            kernels = [k for idx in idxs for k in run_times[idx].kernels]
+            if kernels:
+                rec = records_from_kernels(kernels, dest_device, self._kernel_metadata, mode)
+                res = wave_scale(rec, origin, [dest_device], waves=False)
+                t = res.time_ns[0].cpu().numpy()
+                st = res.status[0].cpu().numpy()
+                bad = np.flatnonzero(st)
+                if bad.size:
+                    raise_for_status(int(st[bad[0]]))
+            pos = 0
+            for idx in idxs:
+                ks = run_times[idx].kernels
+                vals = []
+                for j, k in enumerate(ks):
+                    v = float(t[pos + j])
+                    vals.append(k.run_time_ns if v == k.run_time_ns else v)
+                times[idx] = vals
+                pos += len(ks)
+        for rt, vals in zip(run_times, times):
+            preds = [PredictedKernel(k, v) for k, v in zip(rt.kernels, vals)]
+            out.append(self._assemble(rt, preds, dest_device))
+        return out
+
+    @staticmethod
+    def _assemble(run_time, predicted_kernels, dest_device):
+        run_time_ns = ms_to_ns(run_time.run_time_ms)
+        overhead_ns = run_time_ns - sum(k.run_time_ns for k in run_time.kernels)
+        return RunTimePrediction(overhead_ns=0 if overhead_ns < 0 else overhead_ns,
+                                 predicted_kernels=predicted_kernels, device=dest_device)
+
+    def _special_scale_many(self, kind, operations, dest_device):
+        """predictor.py:132-148 and the four scalers (:150-283), batched: one MLP
+        launch evaluates every operation on its origin and on the destination."""
+        pred = self._mlp(kind)
+        rows = []
+        dest_feats = get_device_features(dest_device.name, pred.device_params)
+        for op in operations:
+            a = _ARGUMENTS[kind](op)
+            feats = [a[x] for x in pred.model.features]
+            rows.append(feats + dest_feats)
+            rows.append(feats + get_device_features(op.device.name, pred.device_params))
+        y = pred.predict_batch(np.asarray(rows, np.float64)).cpu().numpy().astype(np.float64)
+        out = []
+        for i, op in enumerate(operations):
+            ms = op.run_time_ms * float(y[2 * i]) / float(y[2 * i + 1])
+            if ms < 0:
+                logger.warning("Operation %s predicted run time %.2f ms", op.name, ms)
+                ms = 0.
+            out.append(ms)
+        return out
+
+    # scalar faces kept for callers of the reference's private helpers
+    def _special_scale(self, operation, dest_device, scaler):
+        ms = scaler(operation, dest_device)
+        if ms < 0:
+            logger.warning("Operation %s predicted run time %.2f ms", operation.name, ms)
+            ms = 0.
+        return PredictedOperation(operation, RunTimePurePrediction(ms, dest_device), None,
+                                  dest_device)
+
+    def _scale_with(self, kind, operation, dest_device):
+        pred = self._mlp(kind)
+        a = _ARGUMENTS[kind](operation)
+        feats = [a[x] for x in pred.model.features]
+        pred_dest = pred.predict(feats, dest_device.name)
+        pred_orig = pred.predict(feats, operation.device.name)
+        return operation.run_time_ms * pred_dest / pred_orig
+
+    def _conv2d_scale(self, operation, dest_device):
+        return self._scale_with("conv2d", operation, dest_device)
+
+    def _linear_scale(self, operation, dest_device):
+        return self._scale_with("linear", operation, dest_device)
+
+    def _bmm_scale(self, operation, dest_device):
+        return self._scale_with("bmm", operation, dest_device)
+
+    def _lstm_scale(self, operation, dest_device):
+        return self._scale_with("lstm", operation, dest_device)
+
+    # ------------------------------------------------------- device sweeps
+    def predict_trace_times(self, trace, dest_devices):
+        """Predicted iteration time [ms] of `trace` on every device of
+        `dest_devices` (the sum of analysis/trace.py:27-36 over predicted
+        operations).  Kernel records are scaled for all destinations at once."""
+        from habitat_amd.analysis.sweep import predict_trace_times
+        return predict_trace_times(self, trace, dest_devices)

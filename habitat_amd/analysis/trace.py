@@ -1,0 +1,50 @@
+"""An iteration trace: the operations measured on one device, and its
+prediction for another (analyzer/habitat/analysis/trace.py:5-51).
+
+Unlike the reference, importing this module needs no data files: the default
+predictor is built on first use.
+"""
+from habitat_amd.analysis.predictor import Predictor
+
+
+class Trace:
+    _default_predictor = None
+
+    def __init__(self, device, operations):
+        self._device = device
+        self._operations = operations
+        self._run_time_ms = None
+
+    @classmethod
+    def default_predictor(cls):
+        if cls._default_predictor is None:
+            cls._default_predictor = Predictor()
+        return cls._default_predictor
+
+    @property
+    def operations(self):
+        return self._operations
+
+    @property
+    def device(self):
+        return self._device
+
+    @property
+    def run_time_ms(self):
+        if self._run_time_ms is None:
+            self._run_time_ms = sum(op.run_time_ms for op in self._operations)
+        return self._run_time_ms
+
+    def to_device(self, dest_device, predictor=None):
+        """The predicted trace on `dest_device` (all kernels of the trace are
+        scaled in one GPU launch, all MLP operations of a kind in one more)."""
+        if dest_device.name == self.device.name:
+            return self
+        predictor = predictor if predictor is not None else Trace.default_predictor()
+        return Trace(dest_device, predictor.predict_operations(self._operations, dest_device))
+
+    def to_devices(self, dest_devices, predictor=None):
+        """Predicted run time [ms] of the whole trace on each device of a sweep,
+        computed on the GPU; returns a list of floats."""
+        predictor = predictor if predictor is not None else Trace.default_predictor()
+        return predictor.predict_trace_times(self, dest_devices)

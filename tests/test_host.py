@@ -1,0 +1,204 @@
+"""CPU: the C-ABI library loads, exports every symbol include/habitat_mi.h
+declares, and its host-side logic (device specs, host occupancy, argument
+checks) behaves.  No GPU compute is attempted."""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+from conftest import GOLDEN, ROOT
+from habitat_amd import Device, DeviceProperties, _lib, synthetic
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "habitat_mi.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(hbt_[a-z0-9_]+)\s*\(", header))
+    assert {"hbt_wave_scale", "hbt_mlp_forward", "hbt_occupancy_host"} <= declared
+    assert declared == set(_lib.exported_symbols())
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(handle, name), name
+    assert _lib.lib().hbt_version() == 100
+    assert _lib.strerror(0) == "ok" and "spec" in _lib.strerror(_lib.HBT_ESPEC)
+
+
+def test_device_table_and_properties():
+    v100 = Device.V100
+    assert repr(v100) == "DeviceProperties(name=V100)"
+    assert (v100.name, v100.num_sms, v100.mem_bandwidth_gb, v100.compute_capability,
+            v100.base_clock_mhz, v100.peak_gflops_per_second) == ("V100", 80, 739, (7, 0), 1312, 6716)
+    assert set(Device.names()) >= {"P4000", "GTX1080Ti", "RTX2070", "RTX2080Ti", "P4", "T4", "V100",
+                                   "P100", "MI355X"}
+    with pytest.raises(AttributeError):
+        v100.num_sms = 3                      # read-only, as the pybind properties are
+    with pytest.raises(KeyError):
+        Device.NoSuchGPU
+    kw = v100.as_dict()
+    with pytest.raises(TypeError):
+        DeviceProperties(name="x", **dict(kw, num_sms=80.5))
+    with pytest.raises(TypeError):
+        DeviceProperties(name="x", **dict(kw, shared_mem_per_block=-1))   # size_t in the reference
+    with pytest.raises(TypeError):
+        DeviceProperties(**kw)                # name is required
+
+
+def test_host_occupancy_matches_reference_golden(occupancy_golden):
+    g, devices = occupancy_golden
+    rec = dict(block_size=g["block"], dynamic_smem=g["dyn"], static_smem=g["stat"],
+               regs_per_thread=g["regs"])
+    for name, props in devices.items():
+        dev = DeviceProperties(name=name, **props)
+        assert np.array_equal(synthetic.host_occupancy(dev, rec), g["occ_own__" + name]), name
+        # the scalar entry, on a sample
+        for i in range(0, g["block"].shape[0], 401):
+            assert dev.thread_block_occupancy(int(g["block"][i]), int(g["dyn"][i]), int(g["stat"][i]),
+                                              int(g["regs"][i])) == g["occ_own__" + name][i]
+
+
+def test_kernel_instance_occupancy_known_answers(kat):
+    from habitat_amd.analysis.kernels import KernelInstance
+    for dev, block, regs, stat, dyn, occ, _ in kat["occupancy"]:
+        k = KernelInstance("k", 1, block, dyn, stat, regs, 1000)
+        assert k.thread_block_occupancy(getattr(Device, dev)) == occ
+    k = KernelInstance("k", 1, 256, 0, 0, 32, 1000)
+    assert k.thread_block_occupancy(Device.V100, 128) == 2     # explicit register count
+    assert k.thread_block_occupancy(Device.V100, -1) == 8      # negative = own
+    assert k.metadata == {"name": "k", "num_blocks": 1, "block_size": 256,
+                          "static_shared_memory": 0, "dynamic_shared_memory": 0,
+                          "registers_per_thread": 32}
+
+
+def test_spec_check_and_argument_errors():
+    L = _lib.lib()
+    ok = Device.V100.spec
+    assert L.hbt_device_spec_check(ctypes.byref(ok)) == 0
+    assert L.hbt_device_spec_check(None) == _lib.HBT_EINVAL
+    for field, value in (("mem_bandwidth_gb", 0.0), ("base_clock_mhz", float("nan")),
+                         ("peak_gflops", -1.0), ("warp_size", 1 << 16), ("smem_per_sm", -1),
+                         ("num_sms", 1 << 27)):
+        s = _lib.DeviceSpec.from_buffer_copy(ok)
+        setattr(s, field, value)
+        assert L.hbt_device_spec_check(ctypes.byref(s)) == _lib.HBT_ESPEC, field
+    # a device the occupancy model rejects is still a valid spec: occupancy 0
+    s = _lib.DeviceSpec.from_buffer_copy(ok)
+    s.compute_major = 8
+    assert L.hbt_device_spec_check(ctypes.byref(s)) == 0
+    out = ctypes.c_uint32(7)
+    assert L.hbt_occupancy_host(ctypes.byref(s), 256, 0, 0, 32, ctypes.byref(out)) == 0
+    assert out.value == 0
+    assert L.hbt_occupancy_host(None, 256, 0, 0, 32, ctypes.byref(out)) == _lib.HBT_EINVAL
+    # wave scaling: argument checks come before any GPU work
+    z = None
+    rc = L.hbt_wave_scale(ctypes.byref(ok), ctypes.byref(ok), 1, -1, *([z] * 17), None)
+    assert rc == _lib.HBT_EINVAL
+    rc = L.hbt_wave_scale(ctypes.byref(ok), ctypes.byref(ok), 1, 0, *([z] * 17), None)
+    assert rc == 0                                            # nothing to do
+    rc = L.hbt_wave_scale(ctypes.byref(ok), ctypes.byref(ok), 1, 4, *([z] * 17), None)
+    assert rc == _lib.HBT_EINVAL                              # null columns
+    err = ctypes.c_int(0)
+    assert not L.hbt_mlp_create(12, 1024, 8, None, None, None, None, ctypes.byref(err))
+    assert err.value == _lib.HBT_EINVAL
+
+
+def test_compute_entry_fails_loudly_without_gpu():
+    L = _lib.lib()
+    if L.hbt_device_count() > 0:
+        pytest.skip("a GPU is present")
+    ok = Device.V100.spec
+    buf = (ctypes.c_double * 8)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    rc = L.hbt_wave_scale(ctypes.byref(ok), ctypes.byref(ok), 1, 1, p, p, p, p, p, None, p, p, p, p,
+                          None, p, None, None, None, None, None, None)
+    assert rc == _lib.HBT_EHIP
+
+
+def test_synthetic_generators_are_seeded_and_respect_the_origin():
+    rec, stats = synthetic.kernel_records(5000, Device.V100, seed=0)
+    rec2, _ = synthetic.kernel_records(5000, Device.V100, seed=0)
+    assert all(np.array_equal(rec[k], rec2[k]) for k in rec)
+    assert stats["used"] == 5000 and stats["rejected"] > 0
+    assert synthetic.host_occupancy(Device.V100, rec).min() >= 1
+    assert rec["num_blocks"].min() >= 1 and rec["num_blocks"].max() <= 2 ** 20
+    assert set(np.unique(rec["block_size"])) <= {64, 128, 256, 512, 1024}
+    assert rec["run_time_ns"].min() >= 1e3 and rec["run_time_ns"].max() <= 1e7
+    assert np.all(rec["run_time_ns"] == np.floor(rec["run_time_ns"]))
+    devs, feats = synthetic.device_sweep(16, seed=1)
+    assert len(devs) == 16 and feats.shape == (16, 4)
+    assert all(40 <= d.num_sms <= 304 and 500 <= d.mem_bandwidth_gb <= 8000 for d in devs)
+    for kind, f in (("conv2d", 12), ("linear", 8), ("bmm", 8), ("lstm", 11)):
+        x, mu, sigma = synthetic.mlp_features(kind, 256, seed=2)
+        assert x.shape == (256, f) and mu.shape == (f,) and np.all(sigma > 0)
+
+
+def test_mlp_device_features_table():
+    from habitat_amd.analysis.mlp import devices as md
+    assert md.get_device_features("V100", ["mem", "mem_bw", "num_sm", "single"]) == [16, 900, 80, 14.028]
+    assert md.get_device_features("P4000", ["single"]) == [5.3]
+    with pytest.raises(IndexError):
+        md.get_device_features("nope", ["mem"])
+    assert set(md.get_all_devices(["mem"])) >= {"P100", "P4000", "RTX2070", "RTX2080Ti", "T4", "V100"}
+
+
+def test_metrics_and_measured_kernel():
+    from habitat_amd.analysis.kernels import KernelInstance, MeasuredKernel
+    from habitat_amd.analysis.metrics import Metric, resolve_metrics
+    k = KernelInstance("k", 10, 128, 0, 0, 32, 5000)
+    m = KernelInstance("k", 10, 128, 0, 0, 32, 5000, metrics=[("dram_read_bytes", 1e6)])
+    m2 = KernelInstance("k", 10, 128, 0, 0, 32, 5000, metrics=[("dram_utilization", 3.0)])
+    mk = MeasuredKernel(k, [m, m2], Device.P100)
+    assert mk.get_metric(Metric.DRAMReadBytes) == 1e6
+    assert mk.get_metric(Metric.DRAMUtilization) == 30.0          # legacy scale on cc < 7
+    assert mk.get_metric(Metric.DRAMWriteBytes, default=5.0) == 5.0
+    with pytest.raises(AttributeError, match="Unknown metric: DRAMWriteBytes"):
+        mk.get_metric(Metric.DRAMWriteBytes)
+    assert (mk.name, mk.num_blocks, mk.run_time_ns) == ("k", 10, 5000)   # delegated
+    assert resolve_metrics(Metric.DRAMReadBytes, Device.V100) == ["dram__bytes_read.sum"]
+    assert resolve_metrics([Metric.DRAMReadBytes, "raw"], Device.P100) == ["dram_read_bytes", "raw"]
+
+
+def test_habitat_alias_imports():
+    import habitat_amd
+    habitat_amd.install_as_habitat()
+    from habitat.analysis.wave_scaling.common import calculate_wave_info
+    from habitat.analysis.wave_scaling.metadata import MetadataManager  # noqa: F401
+    from habitat.analysis.wave_scaling.resimplified import resimplified_wave_scaling  # noqa: F401
+    from habitat.analysis.wave_scaling.roofline import roofline_wave_scaling  # noqa: F401
+    from habitat.analysis.wave_scaling.unified import unified_wave_scaling  # noqa: F401
+    from habitat.analysis.mlp.mlp import RuntimePredictor, LinearMLP, LSTMMLP, Conv2DMLP, BMMMLP  # noqa: F401
+    from habitat.analysis.predictor import Predictor  # noqa: F401
+    from habitat.analysis.kernels import MeasuredKernel, PredictedKernel, KernelInstance
+    from habitat.analysis.metrics import Metric  # noqa: F401
+    from habitat.analysis.wave_scaling.metadata import NullMetadataManager
+    import habitat
+    assert habitat.Device.V100.num_sms == 80
+    k = KernelInstance("k", 4096, 256, 0, 0, 32, 1000000)
+    assert calculate_wave_info(k, habitat.Device.V100, habitat.Device.P100,
+                               NullMetadataManager()) == (640, 448, 8, 8)
+    assert RuntimePredictor("conv2d", 8, 1024).model.features == [
+        "bias", "batch", "image_size", "in_channels", "out_channels", "kernel_size", "stride",
+        "padding"]
+
+
+def test_metadata_manager_sqlite(tmp_path):
+    import sqlite3
+    from habitat_amd.analysis.kernels import KernelInstance
+    from habitat_amd.analysis.wave_scaling.metadata import MetadataManager
+    path = str(tmp_path / "kernels.sqlite")
+    con = sqlite3.connect(path)
+    con.execute("CREATE TABLE kernels (name TEXT, arch INTEGER, registers_per_thread INTEGER)")
+    con.executemany("INSERT INTO kernels VALUES (?, ?, ?)",
+                    [("gemm", 60, 96), ("gemm", 70, 128), ("relu", 75, 16)])
+    con.commit()
+    con.close()
+    mm = MetadataManager(path)
+    gemm = KernelInstance("gemm", 1, 256, 0, 0, 64, 1)
+    relu = KernelInstance("relu", 1, 256, 0, 0, 64, 1)
+    assert mm.kernel_registers_for(gemm, Device.V100) == 128
+    assert mm.kernel_registers_for(gemm, Device.P4000) == 96      # nearest arch below 61
+    assert mm.kernel_registers_for(gemm, Device.T4) == 128        # 70 <= 75
+    assert mm.kernel_registers_for(relu, Device.V100) is None     # only a newer arch listed
+    assert mm.registers_for_names(["gemm", "relu", "x"], Device.T4) == [128, 16, -1]

@@ -1,0 +1,185 @@
+"""GPU: the fused MFMA MLP (through the C ABI) against the CPU oracle.
+fp32 outputs within 1e-4 relative of the fp64 evaluation of the same weights
+(floor 1e-3 on |reference| for outputs near zero), and no further from it than
+a small multiple of what torch-CPU fp32 — the reference's own arithmetic — is."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import GOLDEN
+from habitat_amd import synthetic
+from habitat_amd.analysis.mlp.mlp import RuntimePredictor
+from oracle import mlp as omlp
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-4
+ABS_FLOOR = 1e-3
+
+
+def assert_close(y, y64, floor=ABS_FLOOR):
+    err = np.abs(y.astype(np.float64) - y64)
+    assert np.all(err <= RTOL * np.maximum(np.abs(y64), floor)), float(err.max())
+
+
+def make(kind, seed=0, hidden=8):
+    torch.manual_seed(seed)
+    rp = RuntimePredictor(kind, hidden, 1024)
+    return rp
+
+
+@pytest.mark.parametrize("kind", ["conv2d", "linear", "bmm", "lstm"])
+def test_seed0_network_4096_rows(kind):
+    rp = make(kind)
+    sd = rp.model.state_dict()
+    with open(os.path.join(GOLDEN, "mlp_seed0.json")) as f:
+        g = json.load(f)[kind]
+    assert omlp.state_dict_sha256(sd) == g["sha256"]
+    x, mu, sigma = synthetic.mlp_features(kind, 4096, seed=2)
+    rp.set_normalization(mu, sigma)
+    y = rp.predict_batch(x).cpu().numpy()
+    y64 = omlp.forward_fp64(sd, x, mu, sigma)
+    y32 = omlp.forward_fp32(sd, x, mu, sigma)
+    assert_close(y, y64)
+    assert np.max(np.abs(y - y64)) <= 8 * max(np.max(np.abs(y32 - y64)), 1e-8)
+    # committed golden rows
+    assert_close(y[:16], np.array(g["fp64"]))
+
+
+def test_trained_like_weights_with_wide_output_range():
+    # Random-init outputs barely move; scale the layers and centre the output so
+    # that predictions spread over several units and change sign, which is what
+    # exercises cancellation in the last dot product.
+    rp = make("conv2d", seed=7)
+    with torch.no_grad():
+        for name, p in rp.model.named_parameters():
+            if name.endswith("weight"):
+                p.mul_(2.5)
+            else:
+                p.add_(0.05 * torch.randn_like(p))
+        rp.model.fc2.weight.copy_(torch.randn(1, 1024) * 0.05)
+        rp.model.fc2.bias.fill_(-1.5)
+    x, mu, sigma = synthetic.mlp_features("conv2d", 8192, seed=21)
+    rp.set_normalization(mu, sigma)
+    sd = rp.model.state_dict()
+    y = rp.predict_batch(x).cpu().numpy()
+    y64 = omlp.forward_fp64(sd, x, mu, sigma)
+    assert y64.max() - y64.min() > 1.0 and y64.min() < 0 < y64.max()
+    # Outputs near zero are differences of terms of size |fc2.bias| = 1.5: the
+    # relative bound is taken against that magnitude there, and the error must
+    # stay within a small multiple of what torch-CPU fp32 itself makes.
+    assert_close(y, y64, floor=1.5)
+    y32 = omlp.forward_fp32(sd, x, mu, sigma)
+    assert np.max(np.abs(y - y64)) <= 4 * np.max(np.abs(y32 - y64))
+
+
+@pytest.mark.parametrize("n", [1, 2, 31, 32, 33, 63, 65, 1000])
+def test_ragged_row_counts(n):
+    rp = make("lstm")
+    x, mu, sigma = synthetic.mlp_features("lstm", 1000, seed=5)
+    rp.set_normalization(mu, sigma)
+    y = rp.predict_batch(x[:n]).cpu().numpy()
+    assert y.shape == (n,)
+    assert_close(y, omlp.forward_fp64(rp.model.state_dict(), x[:n], mu, sigma))
+
+
+def test_empty_batch():
+    rp = make("bmm")
+    rp.set_normalization(np.zeros(8), np.ones(8))
+    assert rp.predict_batch(np.zeros((0, 8))).shape == (0,)
+
+
+def test_exact_cases_dead_relu_and_selector_weights():
+    rp = make("linear", hidden=2)
+    x, mu, sigma = synthetic.mlp_features("linear", 200, seed=6)
+    rp.set_normalization(mu, sigma)
+    with torch.no_grad():
+        rp.model.mlp.layers[2].bias.fill_(-1e6)
+    rp.refresh()
+    y = rp.predict_batch(x).cpu().numpy()
+    assert np.all(y == rp.model.fc2.bias.item())          # every ReLU dead: exact
+    # Selector network: fc1 copies feature j to unit j (plus 100 so ReLU stays open),
+    # hidden layers are identities, fc2 picks unit `pick` -> out = x_std[pick] + 100.
+    with torch.no_grad():
+        for p in rp.model.parameters():
+            p.zero_()
+        for j in range(8):
+            rp.model.fc1.weight[j, j] = 1.0
+        rp.model.fc1.bias[:8] = 100.0
+        for layer in (rp.model.mlp.layers[0], rp.model.mlp.layers[2]):
+            layer.weight.copy_(torch.eye(1024))
+    for pick in (0, 3, 7):
+        with torch.no_grad():
+            rp.model.fc2.weight.zero_()
+            rp.model.fc2.weight[0, pick] = 1.0
+        rp.refresh()
+        y = rp.predict_batch(x).cpu().numpy()
+        want = (omlp.standardise(x, mu, sigma)[:, pick] + np.float32(100.0)).astype(np.float32)
+        assert np.array_equal(y, want), pick
+
+
+def test_every_weight_position_is_wired():
+    # One hidden layer holding a random permutation matrix scaled by distinct
+    # powers of two: out[r] = sum over units of 2^-(j%8) * in[perm[j]] exactly
+    # representable, so a mis-packed weight shows up as a wrong value.
+    rp = make("bmm", hidden=1)
+    rng = np.random.default_rng(3)
+    perm = rng.permutation(1024)
+    with torch.no_grad():
+        for p in rp.model.parameters():
+            p.zero_()
+        w1 = torch.zeros(1024, 8)
+        for j in range(1024):
+            w1[j, j % 8] = float(1 + (j // 8) % 4)
+        rp.model.fc1.weight.copy_(w1)
+        rp.model.fc1.bias.fill_(64.0)
+        wh = torch.zeros(1024, 1024)
+        for j in range(1024):
+            wh[j, perm[j]] = 2.0 ** -(j % 8)
+        rp.model.mlp.layers[0].weight.copy_(wh)
+        rp.model.fc2.weight.copy_(torch.from_numpy(
+            (rng.integers(0, 2, 1024) * 2 - 1).astype(np.float32))[None])
+    rp.set_normalization(np.zeros(8), np.ones(8))
+    x = rng.integers(-4, 5, size=(96, 8)).astype(np.float64)   # small integers: exact sums
+    y = rp.predict_batch(x).cpu().numpy()
+    y64 = omlp.forward_fp64(rp.model.state_dict(), x, np.zeros(8), np.ones(8))
+    assert np.array_equal(y.astype(np.float64), y64)
+
+
+def test_scalar_predict_and_checkpoint_round_trip(tmp_path):
+    rp = make("conv2d")
+    x, mu, sigma = synthetic.mlp_features("conv2d", 64, seed=2)
+    rp.set_normalization(mu, sigma)
+    path = str(tmp_path / "model.pth")
+    rp.save_state(path)
+    rp2 = RuntimePredictor("conv2d", 8, 1024, path)
+    assert np.array_equal(rp2.mu, mu)
+    args = [1, 32, 56, 64, 128, 3, 1, 1]
+    a, b = rp.predict(args, "V100"), rp2.predict(args, "V100")
+    assert isinstance(a, float) and a == b
+    row = np.array([args + [16, 900, 80, 14.028]], np.float64)
+    assert_close(np.array([a], np.float32), omlp.forward_fp64(rp.model.state_dict(), row, mu, sigma))
+    with pytest.raises(IndexError):
+        rp.predict(args, "UnknownGPU")
+    with pytest.raises(TypeError):
+        RuntimePredictor("conv2d", 8, 1024).predict(args, "V100")     # no mu/sigma
+
+
+def test_config2_full_size_properties():
+    # 1M rows: the oracle is too slow for all of them, so check a strided
+    # sample against it and, over the whole batch, invariance to row order.
+    rp = make("conv2d")
+    n = 1_000_000
+    x, mu, sigma = synthetic.mlp_features("conv2d", n, seed=2)
+    rp.set_normalization(mu, sigma)
+    xg = torch.from_numpy(x).cuda()
+    y = rp.predict_batch(xg)
+    idx = np.arange(0, n, 997)
+    assert_close(y.cpu().numpy()[idx], omlp.forward_fp64(rp.model.state_dict(), x[idx], mu, sigma))
+    perm = torch.randperm(n, device="cuda", generator=torch.Generator("cuda").manual_seed(1))
+    y_perm = rp.predict_batch(xg[perm].contiguous())
+    assert torch.equal(y_perm, y[perm])          # a row's result does not depend on its neighbours
+    assert bool(torch.all(torch.isfinite(y)))

@@ -1,0 +1,230 @@
+"""CPU: pins the oracle (oracle/occupancy.c, wave_scaling.c, wave_scaling.py)
+before anything is compared with it: reference-compiled golden vectors,
+hand-derived known answers, the compiled reference itself where it was built,
+closed forms and invariants."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+from conftest import GOLDEN, oracle_device
+from oracle import lib as olib
+from oracle import wave_scaling as ows
+
+
+def _devs():
+    with open(os.path.join(GOLDEN, "occupancy_golden_devices.json")) as f:
+        return json.load(f)
+
+
+DEVS = _devs()
+
+
+# ----------------------------------------------------------------- occupancy
+def test_oracle_occupancy_matches_reference_golden(occupancy_golden):
+    g, devices = occupancy_golden
+    assert g["block"].shape[0] > 12000 and len(devices) >= 12
+    for name, props in devices.items():
+        d = oracle_device(props)
+        own = olib.occupancy_batch(d, g["block"], g["dyn"], g["stat"], g["regs"])
+        lut = olib.occupancy_batch(d, g["block"], g["dyn"], g["stat"], g["regs"], g["dregs"])
+        assert np.array_equal(own, g["occ_own__" + name]), name
+        assert np.array_equal(lut, g["occ_lut__" + name]), name
+
+
+def test_oracle_occupancy_matches_compiled_reference_on_fresh_inputs():
+    if olib.ref() is None:
+        pytest.skip("oracle/_ref was not built (reference tree not mounted)")
+    rng = np.random.default_rng(99)
+    n = 50000
+    block = rng.integers(1, 1100, n).astype(np.int32)
+    dyn = rng.integers(0, 70000, n).astype(np.int32)
+    stat = rng.integers(0, 50000, n).astype(np.int32)
+    regs = rng.integers(0, 300, n).astype(np.int32)
+    for name, props in DEVS.items():
+        d = oracle_device(props)
+        assert np.array_equal(olib.occupancy_batch(d, block, dyn, stat, regs),
+                              olib.ref_occupancy_batch(d, block, dyn, stat, regs)), name
+
+
+def test_oracle_occupancy_known_answers(kat):
+    for dev, block, regs, stat, dyn, occ, wave in kat["occupancy"]:
+        d = oracle_device(DEVS[dev])
+        got = olib.occupancy(d, block, dyn, stat, regs)
+        assert got == occ, (dev, block, regs, stat, dyn)
+        if wave is not None:
+            assert got * d.num_sms == wave
+    for row in kat["occupancy_limits"]:
+        d = oracle_device(DEVS[row["device"]])
+        occ, lim = olib.occupancy_limits(d, row["block"], row["smem"], 0, row["regs"])
+        assert (lim.regs, lim.warps, lim.blocks, lim.smem) == (
+            row["reg"], row["warp"], row["block_slots"], row["smem_limit"]), row
+        assert occ == min(lim.regs, lim.warps, lim.blocks, lim.smem)
+
+
+def test_oracle_occupancy_invariants():
+    rng = np.random.default_rng(5)
+    d = oracle_device(DEVS["V100"])
+    for _ in range(300):
+        block = int(rng.integers(1, 1025))
+        smem = int(rng.integers(0, 49152))
+        regs = int(rng.integers(0, 200))
+        occ, lim = olib.occupancy_limits(d, block, smem, 0, regs)
+        assert occ == min(lim.regs, lim.warps, lim.blocks, lim.smem)
+        # more registers or more shared memory never raise the occupancy
+        assert olib.occupancy(d, block, smem, 0, regs + 8) <= occ
+        assert olib.occupancy(d, block, smem + 1024, 0, regs) <= occ
+        # nothing but warps and block slots limit a kernel without resources
+        assert olib.occupancy(d, block, 0, 0, 0) == min(lim.warps, lim.blocks)
+    # 16-bit narrowing of the register count (kernel.h:108)
+    assert olib.occupancy(d, 256, 0, 0, 65536 + 32) == olib.occupancy(d, 256, 0, 0, 32)
+
+
+# -------------------------------------------------------------- wave scaling
+def _record(kat, num_blocks, **over):
+    rec = dict(kat["scaling_record"], num_blocks=num_blocks)
+    rec.update(over)
+    return rec
+
+
+def _cols(recs):
+    return {k: np.array([r[k] for r in recs]) for k in recs[0]}
+
+
+def test_scaling_known_answers_python_and_c(kat):
+    for row in kat["scaling"]:
+        o, d = oracle_device(DEVS[row["origin"]]), oracle_device(DEVS[row["dest"]])
+        rec = _record(kat, row["num_blocks"])
+        assert ows.gamma(rec, o, d) == pytest.approx(row["gamma"], rel=1e-15)
+        assert ows.unified(rec, o, d) == pytest.approx(row["time_ns"], rel=1e-14)
+        c = olib.wave_scale(o, d, _cols([rec]), want_gamma=True)
+        assert c["status"][0] == 0
+        assert c["time_ns"][0] == pytest.approx(row["time_ns"], rel=1e-14)
+        assert c["gamma"][0] == pytest.approx(row["gamma"], rel=1e-15)
+        wave_o, wave_d, _, _ = ows.wave_info(rec, o, d)
+        small = row["num_blocks"] < wave_o and row["num_blocks"] < wave_d
+        assert small == (row["branch"] == "small")
+
+
+def test_scaling_closed_forms(kat):
+    v100, p100 = oracle_device(DEVS["V100"]), oracle_device(DEVS["P100"])
+    big = 1 << 16
+    # same device on both sides: identity on both strategies and both branches
+    for nb in (3, big):
+        for hm in (True, False):
+            t = ows.unified(_record(kat, nb), v100, v100, has_metrics=hm)
+            assert t == pytest.approx(1e6, rel=1e-15)
+    # no FLOPs: gamma = 1, pure bandwidth ratio
+    t = ows.unified(_record(kat, big, flop_sp_efficiency=0.0), v100, p100)
+    assert ows.gamma(_record(kat, big, flop_sp_efficiency=0.0), v100, p100) == 1.0
+    assert t == pytest.approx(1e6 * 739 / 501, rel=1e-15)
+    # no bytes but FLOPs: gamma = 0, clock ratio times SM ratio
+    r = _record(kat, big, dram_read_bytes=0.0, dram_write_bytes=0.0)
+    assert ows.gamma(r, v100, p100) == 0.0
+    assert ows.unified(r, v100, p100) == pytest.approx(1e6 * (1312 / 1126) * (80 / 56), rel=1e-15)
+    # intensity exactly at the ridge point: both formulas give 1/2
+    ridge = 9504 / 501
+    gflops = 50.0 / 100 * 6716 * 1e6 / 1e9
+    nbytes = gflops / ridge * 1024 ** 3
+    r_lo = _record(kat, big, dram_read_bytes=nbytes * (1 + 1e-9), dram_write_bytes=0.0)
+    r_hi = _record(kat, big, dram_read_bytes=nbytes * (1 - 1e-9), dram_write_bytes=0.0)
+    assert ows.gamma(r_lo, v100, p100) == pytest.approx(0.5, abs=1e-8)
+    assert ows.gamma(r_hi, v100, p100) == pytest.approx(0.5, abs=1e-8)
+    # without metrics: small kernel unchanged, else bandwidth ratio
+    assert ows.unified(_record(kat, 3), v100, p100, has_metrics=False) == 1000000
+    assert ows.unified(_record(kat, big), v100, p100, has_metrics=False) == pytest.approx(
+        1e6 * 739 / 501, rel=1e-15)
+    # destination register count from the look-up table changes the wave size only
+    r = _record(kat, 500)
+    assert ows.wave_info(r, v100, p100, dest_regs=128)[3] == 2
+    assert ows.wave_info(r, v100, p100)[3] == 8
+
+
+def test_scaling_exceptions_and_statuses(kat):
+    v100, p100, mi = (oracle_device(DEVS[k]) for k in ("V100", "P100", "MI355X"))
+    cases = [
+        # origin cannot hold the block at all
+        (_record(kat, 100, regs_per_thread=255, block_size=1024), v100, p100, True, 1),
+        # destination occupancy 0 and the kernel is small on the origin
+        (_record(kat, 10, dynamic_smem=60000), mi, v100, True, 2),
+        (_record(kat, 10, dynamic_smem=60000), mi, v100, False, 2),
+        # ... but not evaluated when the origin test already fails (big kernel)
+        (_record(kat, 1 << 16, dynamic_smem=60000), mi, v100, True, 0),
+        (_record(kat, 1 << 16, dynamic_smem=60000), mi, v100, False, 0),
+        # negative byte counts push gamma above 1
+        (_record(kat, 100, dram_read_bytes=-3e8), v100, p100, True, 3),
+        (_record(kat, 100, flop_sp_efficiency=float("nan")), v100, p100, True, 3),
+        # a bad gamma is found before a zero wave size
+        (_record(kat, 100, regs_per_thread=255, block_size=1024, dram_read_bytes=-3e8),
+         v100, p100, True, 3),
+        # num_blocks 0: ceil(0 / sms) = 0 divides
+        (_record(kat, 0), v100, p100, True, 4),
+        (_record(kat, 0), v100, p100, False, 0),
+        # negative num_blocks is never "small" (floor division gives -1)
+        (_record(kat, -5), v100, p100, True, 0),
+    ]
+    for rec, o, d, hm, want in cases:
+        t, st = ows.unified_with_status(rec, o, d, has_metrics=hm)
+        assert st == want, (rec, want)
+        cols = _cols([rec])
+        cols["has_metrics"] = np.array([1 if hm else 0], np.uint8)
+        c = olib.wave_scale(o, d, cols)
+        assert c["status"][0] == want
+        if want:
+            assert math.isnan(c["time_ns"][0]) and math.isnan(t)
+            with pytest.raises(ows.STATUS_EXCEPTION[want]):
+                ows.unified(rec, o, d, has_metrics=hm)
+        else:
+            assert c["time_ns"][0] == t
+
+
+def test_c_restatement_equals_python_restatement_bit_for_bit():
+    rng = np.random.default_rng(11)
+    n = 3000
+    recs = []
+    for _ in range(n):
+        total = int(rng.integers(0, 65537))
+        recs.append(dict(
+            num_blocks=int(2 ** rng.uniform(0, 20)), block_size=int(rng.choice([64, 128, 256, 512, 1024])),
+            dynamic_smem=total - total // 2, static_smem=total // 2,
+            regs_per_thread=int(rng.integers(16, 256)), run_time_ns=float(int(10 ** rng.uniform(3, 7))),
+            flop_sp_efficiency=float(10 ** rng.uniform(-2, 2)),
+            dram_read_bytes=float(int(10 ** rng.uniform(3, 10))),
+            dram_write_bytes=float(int(10 ** rng.uniform(3, 10)))))
+    cols = _cols(recs)
+    hm = (rng.random(n) < 0.7).astype(np.uint8)
+    dr = np.where(rng.random(n) < 0.3, rng.integers(16, 200, n), -1).astype(np.int32)
+    cols["has_metrics"], cols["dest_regs"] = hm, dr
+    for on, dn in (("V100", "MI355X"), ("MI355X", "V100"), ("P100", "T4"), ("T4", "P4000")):
+        o, d = oracle_device(DEVS[on]), oracle_device(DEVS[dn])
+        c = olib.wave_scale(o, d, cols)
+        seen = set()
+        for i, rec in enumerate(recs):
+            t, st = ows.unified_with_status(rec, o, d, dest_regs=None if dr[i] < 0 else int(dr[i]),
+                                            has_metrics=bool(hm[i]))
+            assert st == c["status"][i]
+            seen.add(st)
+            if st == 0:
+                assert t == c["time_ns"][i]  # identical doubles
+            else:
+                assert math.isnan(c["time_ns"][i])
+        assert 0 in seen
+
+
+def test_python_restatement_over_compiled_reference_occupancy(kat):
+    """The wave-scaling restatement gives the same answers when its occupancy
+    comes from the reference's own routine."""
+    ref = olib.ref()
+    if ref is None:
+        pytest.skip("oracle/_ref was not built (reference tree not mounted)")
+    import ctypes
+
+    def ref_occ(dev, rec, regs):
+        return int(ref.ref_occupancy(ctypes.byref(dev), rec["block_size"], rec["dynamic_smem"],
+                                     rec["static_smem"], rec["regs_per_thread"], regs))
+    for row in kat["scaling"]:
+        o, d = oracle_device(DEVS[row["origin"]]), oracle_device(DEVS[row["dest"]])
+        rec = _record(kat, row["num_blocks"])
+        assert ows.unified(rec, o, d, occupancy=ref_occ) == pytest.approx(row["time_ns"], rel=1e-14)

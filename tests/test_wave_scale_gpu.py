@@ -1,0 +1,220 @@
+"""GPU: the HIP wave-scaling path (through the C ABI) against the CPU oracle.
+Integers and statuses bit-exact; fp64 times within 1e-6 relative."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import GOLDEN, oracle_device
+from habitat_amd import Device, DeviceProperties, synthetic
+from habitat_amd.analysis.wave_scaling.batch import KernelRecords, WaveScaleOutput, wave_scale
+from oracle import lib as olib
+
+pytestmark = pytest.mark.gpu
+
+TIME_RTOL = 1e-6   # tolerance for the fp64 scaled time
+
+
+def odev(d):
+    return oracle_device(d.as_dict())
+
+
+def check(rec, origin, dests, out, rows=None):
+    """Compare every output of `out` with the oracle."""
+    n = rec["num_blocks"].shape[0]
+    occ_o = out.occ_origin.cpu().numpy()
+    for di, d in enumerate(dests):
+        want = olib.wave_scale(odev(origin), odev(d), rec)
+        assert np.array_equal(occ_o, want["occ_origin"])
+        assert np.array_equal(out.occ_dest[di].cpu().numpy(), want["occ_dest"]), d.name
+        if out.wave_origin is not None:
+            assert np.array_equal(out.wave_origin.cpu().numpy(), want["wave_origin"])
+            assert np.array_equal(out.wave_dest[di].cpu().numpy(), want["wave_dest"])
+        st = out.status[di].cpu().numpy()
+        assert np.array_equal(st, want["status"]), d.name
+        t = out.time_ns[di].cpu().numpy()
+        ok = want["status"] == 0
+        assert np.all(np.isnan(t[~ok]))
+        np.testing.assert_allclose(t[ok], want["time_ns"][ok], rtol=TIME_RTOL, atol=0)
+    return n
+
+
+def test_config0_10k_records_v100_to_mi355x():
+    rec, stats = synthetic.kernel_records(10_000, Device.V100, seed=0)
+    out = wave_scale(KernelRecords.from_numpy(rec), Device.V100, [Device.MI355X])
+    check(rec, Device.V100, [Device.MI355X], out)
+
+
+def test_config1_1m_records():
+    rec, _ = synthetic.kernel_records(1_000_000, Device.V100, seed=0)
+    out = wave_scale(KernelRecords.from_numpy(rec), Device.V100, [Device.MI355X])
+    check(rec, Device.V100, [Device.MI355X], out)
+    # size-independent properties at the full size
+    t = out.time_ns[0]
+    assert bool(torch.all(t > 0)) and bool(torch.all(torch.isfinite(t)))
+    # V100 -> MI355X: every factor favours the destination, so times shrink
+    assert bool(torch.all(t < torch.from_numpy(rec["run_time_ns"]).cuda()))
+
+
+def test_identity_and_round_trip_properties():
+    rec, _ = synthetic.kernel_records(200_000, Device.V100, seed=3, metrics_fraction=0.5)
+    kr = KernelRecords.from_numpy(rec)
+    same = wave_scale(kr, Device.V100, [Device.V100])
+    t = same.time_ns[0].cpu().numpy()
+    np.testing.assert_allclose(t, rec["run_time_ns"], rtol=1e-12)
+    assert np.array_equal(same.occ_origin.cpu().numpy(), same.occ_dest[0].cpu().numpy())
+    # linearity in the measured time: scaling 3t gives 3 * scale(t) unless gamma moves
+    rec3 = dict(rec, flop_sp_efficiency=np.zeros_like(rec["flop_sp_efficiency"]))   # gamma = 1
+    a = wave_scale(KernelRecords.from_numpy(rec3), Device.V100, [Device.T4]).time_ns[0].cpu().numpy()
+    rec3["run_time_ns"] = rec3["run_time_ns"] * 3
+    b = wave_scale(KernelRecords.from_numpy(rec3), Device.V100, [Device.T4]).time_ns[0].cpu().numpy()
+    np.testing.assert_allclose(b, 3 * a, rtol=1e-12)
+
+
+def test_every_device_pair_with_metrics_mix_and_register_table():
+    rng = np.random.default_rng(4)
+    names = ["P4000", "GTX1080Ti", "RTX2070", "RTX2080Ti", "P4", "T4", "V100", "P100", "MI355X"]
+    for oname in ("V100", "P100", "T4", "MI355X", "P4000"):
+        origin = getattr(Device, oname)
+        rec, _ = synthetic.kernel_records(20_000, origin, seed=5, metrics_fraction=0.6)
+        rec["dest_regs"] = np.where(rng.random(20_000) < 0.4, rng.integers(0, 300, 20_000),
+                                    -1).astype(np.int32)
+        dests = [getattr(Device, n) for n in names]          # 9 destinations: two launches
+        out = wave_scale(KernelRecords.from_numpy(rec), origin, dests)
+        check(rec, origin, dests, out)
+
+
+def test_every_status_and_the_short_circuit(kat):
+    base = dict(kat["scaling_record"])
+    rows = [
+        dict(base, num_blocks=100, regs_per_thread=255, block_size=1024),              # 1
+        dict(base, num_blocks=10, dynamic_smem=60000),                                 # 2 (MI355X -> V100)
+        dict(base, num_blocks=1 << 16, dynamic_smem=60000),                            # 0: not evaluated
+        dict(base, num_blocks=100, dram_read_bytes=-3e8),                              # 3
+        dict(base, num_blocks=100, flop_sp_efficiency=float("nan")),                   # 3
+        dict(base, num_blocks=0),                                                      # 4 / 0 without metrics
+        dict(base, num_blocks=-5),                                                     # 0
+        dict(base, num_blocks=100, flop_sp_efficiency=float("inf")),                   # gamma 0+
+        dict(base, num_blocks=100, dram_read_bytes=0.0, dram_write_bytes=0.0),         # gamma 0
+        dict(base, num_blocks=100, flop_sp_efficiency=0.0),                            # gamma 1
+    ]
+    rec = {k: np.array([r[k] for r in rows]) for k in rows[0]}
+    for hm in (1, 0):
+        rec["has_metrics"] = np.full(len(rows), hm, np.uint8)
+        for origin, dest in ((Device.MI355X, Device.V100), (Device.V100, Device.P100)):
+            out = wave_scale(KernelRecords.from_numpy(rec), origin, [dest])
+            check(rec, origin, [dest], out)
+    rec["has_metrics"] = np.ones(len(rows), np.uint8)
+    st = wave_scale(KernelRecords.from_numpy(rec), Device.MI355X, [Device.V100]).status[0].cpu().numpy()
+    assert list(st[:7]) == [1, 2, 0, 3, 3, 4, 0]
+
+
+def test_golden_launch_configurations_on_all_fixture_devices(occupancy_golden):
+    g, devices = occupancy_golden
+    n = g["block"].shape[0]
+    rng = np.random.default_rng(8)
+    rec = {"num_blocks": rng.integers(1, 5000, n).astype(np.int32), "block_size": g["block"],
+           "dynamic_smem": g["dyn"], "static_smem": g["stat"], "regs_per_thread": g["regs"],
+           "dest_regs": g["dregs"], "run_time_ns": np.full(n, 1e5),
+           "flop_sp_efficiency": np.full(n, 20.0), "dram_read_bytes": np.full(n, 1e7),
+           "dram_write_bytes": np.full(n, 1e6)}
+    kr = KernelRecords.from_numpy(rec)
+    names = list(devices)
+    dests = [DeviceProperties(name=k, **devices[k]) for k in names]
+    origin = dests[names.index("V100")]
+    out = wave_scale(kr, origin, dests)
+    for di, name in enumerate(names):
+        # occupancies straight against the reference-compiled fixture
+        assert np.array_equal(out.occ_dest[di].cpu().numpy(), g["occ_lut__" + name]), name
+    assert np.array_equal(out.occ_origin.cpu().numpy(), g["occ_own__V100"])
+    check(rec, origin, dests, out)
+
+
+def test_slow_division_path_with_huge_device_and_record_values():
+    big = DeviceProperties(name="big", **dict(
+        Device.V100.as_dict(), max_threads_per_block=1 << 24, max_threads_per_multiprocessor=1 << 26,
+        regs_per_block=1 << 30, regs_per_multiprocessor=1 << 30,
+        shared_mem_per_block=1 << 28, shared_mem_per_multiprocessor=1 << 29, warp_size=48))
+    rng = np.random.default_rng(10)
+    n = 4096
+    rec = {"num_blocks": rng.integers(1, 1 << 30, n).astype(np.int32),
+           "block_size": rng.integers(1, 1 << 24, n).astype(np.int32),
+           "dynamic_smem": rng.integers(0, 1 << 27, n).astype(np.int32),
+           "static_smem": rng.integers(0, 1 << 27, n).astype(np.int32),
+           "regs_per_thread": rng.integers(0, 256, n).astype(np.int32),
+           "run_time_ns": np.floor(10.0 ** rng.uniform(3, 7, n)),
+           "flop_sp_efficiency": 10.0 ** rng.uniform(-2, 2, n),
+           "dram_read_bytes": np.floor(10.0 ** rng.uniform(3, 10, n)),
+           "dram_write_bytes": np.floor(10.0 ** rng.uniform(3, 10, n))}
+    for origin, dest in ((big, Device.V100), (Device.V100, big), (big, big)):
+        out = wave_scale(KernelRecords.from_numpy(rec), origin, [dest])
+        check(rec, origin, [dest], out)
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 255, 256, 257, 1023, 1025])
+def test_ragged_sizes_single_and_multi_destination(n):
+    rec, _ = synthetic.kernel_records(n, Device.V100, seed=n)
+    dests = [Device.MI355X, Device.T4, Device.P100]
+    kr = KernelRecords.from_numpy(rec)
+    check(rec, Device.V100, dests[:1], wave_scale(kr, Device.V100, dests[:1]))
+    check(rec, Device.V100, dests, wave_scale(kr, Device.V100, dests))
+
+
+def test_empty_input_and_no_destinations():
+    rec, _ = synthetic.kernel_records(8, Device.V100, seed=0)
+    empty = {k: v[:0] for k, v in rec.items()}
+    out = wave_scale(KernelRecords.from_numpy(empty), Device.V100, [Device.T4])
+    assert out.time_ns.shape == (1, 0)
+    out = wave_scale(KernelRecords.from_numpy(rec), Device.V100, [])
+    assert out.time_ns.shape == (0, 8)
+
+
+def test_unaligned_columns_take_the_element_wise_kernel():
+    rec, _ = synthetic.kernel_records(1001, Device.V100, seed=12)
+    shifted = {}
+    for k, v in rec.items():
+        t = torch.from_numpy(np.concatenate([v[:1], v])).cuda()
+        shifted[k] = t[1:]                       # 4- or 8-byte aligned only
+        assert shifted[k].data_ptr() % 16 != 0
+    kr = KernelRecords(shifted)
+    out = wave_scale(kr, Device.V100, [Device.MI355X, Device.P4])
+    check(rec, Device.V100, [Device.MI355X, Device.P4], out)
+
+
+def test_outputs_are_optional_and_buffers_reusable():
+    rec, _ = synthetic.kernel_records(4096, Device.V100, seed=13)
+    kr = KernelRecords.from_numpy(rec)
+    full = wave_scale(kr, Device.V100, [Device.T4])
+    bare = WaveScaleOutput(4096, 1, kr.device, waves=False, status=False)
+    assert bare.wave_dest is None and bare.status is None
+    for _ in range(2):
+        wave_scale(kr, Device.V100, [Device.T4], out=bare)
+    assert torch.equal(bare.time_ns, full.time_ns)
+    assert torch.equal(bare.occ_dest, full.occ_dest)
+    with pytest.raises(ValueError):
+        wave_scale(kr, Device.V100, [Device.T4, Device.P4], out=bare)
+
+
+def test_runs_on_a_side_stream():
+    rec, _ = synthetic.kernel_records(50_000, Device.V100, seed=14)
+    kr = KernelRecords.from_numpy(rec)
+    want = wave_scale(kr, Device.V100, [Device.T4])
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        got = wave_scale(kr, Device.V100, [Device.T4])
+    s.synchronize()
+    assert torch.equal(got.time_ns, want.time_ns)
+
+
+def test_bad_specs_are_rejected_not_launched():
+    from habitat_amd import _lib
+    rec, _ = synthetic.kernel_records(16, Device.V100, seed=0)
+    kr = KernelRecords.from_numpy(rec)
+    zero_bw = DeviceProperties(name="z", **dict(Device.V100.as_dict(), mem_bandwidth_gb=0))
+    with pytest.raises(_lib.HabitatLibraryError) as e:
+        wave_scale(kr, Device.V100, [zero_bw])
+    assert e.value.code == _lib.HBT_ESPEC
