@@ -44,6 +44,8 @@ _SIGNATURES = {
     "hbt_occupancy_host": (C.c_int, [C.POINTER(DeviceSpec), C.c_int32, C.c_int32, C.c_int32,
                                      C.c_int32, C.POINTER(C.c_uint32)]),
     "hbt_occupancy_host_batch": (C.c_int, [C.POINTER(DeviceSpec), C.c_int64, _P, _P, _P, _P, _P]),
+    "hbt_occupancy_host_model32_batch": (C.c_int, [C.POINTER(DeviceSpec), C.c_int64, _P, _P, _P, _P,
+                                                   _P]),
     "hbt_wave_scale": (C.c_int, [C.POINTER(DeviceSpec), C.POINTER(DeviceSpec), C.c_int32,
                                  C.c_int64] + [_P] * 17 + [_P]),
     "hbt_mlp_create": (_P, [C.c_int32, C.c_int32, C.c_int32, C.POINTER(_P), C.POINTER(_P), _P, _P,

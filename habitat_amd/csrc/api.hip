@@ -15,16 +15,24 @@ namespace hbt {
 DestArgs make_dest_args(const hbt_device_spec& o, const hbt_device_spec& d) {
   DestArgs p{};
   p.dev = make_occ_device(d);
-  p.sms = (double)d.num_sms;
+  p.inv_sms = 1.0f / (float)d.num_sms;
   p.ridge = d.peak_gflops / d.mem_bandwidth_gb;
   p.half_ridge = 0.5 * p.ridge;
   p.neg_half_over_ridge = -0.5 / p.ridge;
   p.bw_ratio = o.mem_bandwidth_gb / d.mem_bandwidth_gb;
-  p.clk_ratio = o.base_clock_mhz / d.base_clock_mhz;
+  const double clk_ratio = o.base_clock_mhz / d.base_clock_mhz;
   const double sm_ratio = (double)o.num_sms / (double)d.num_sms;
   p.log2_bw = std::log2(p.bw_ratio);
-  p.log2_clk_sm = std::log2(p.clk_ratio) + std::log2(sm_ratio);
+  p.log2_clk = std::log2(clk_ratio);
+  p.log2_clk_sm = p.log2_clk + std::log2(sm_ratio);
   return p;
+}
+
+// What make_occ_device needs: 32-bit shared-memory sizes and a bounded warp size.
+static bool occupancy_spec_in_domain(const hbt_device_spec& s) {
+  const int64_t two31 = (int64_t)1 << 31;
+  return s.warp_size <= 32768 && s.smem_per_block >= 0 && s.smem_per_block < two31 &&
+         s.smem_per_sm >= 0 && s.smem_per_sm < two31;
 }
 
 static bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
@@ -74,8 +82,7 @@ int hbt_device_spec_check(const hbt_device_spec* s) {
 int hbt_occupancy_host(const hbt_device_spec* spec, int32_t block_size, int32_t dynamic_smem,
                        int32_t static_smem, int32_t regs, uint32_t* out) {
   if (spec == nullptr || out == nullptr) return HBT_EINVAL;
-  if (spec->warp_size > 32768 || spec->smem_per_block < 0 || spec->smem_per_sm < 0)
-    return HBT_ESPEC;
+  if (!hbt::occupancy_spec_in_domain(*spec)) return HBT_ESPEC;
   const hbt::OccDevice d = hbt::make_occ_device(*spec);
   *out = (uint32_t)hbt::occupancy_exact(d, block_size, dynamic_smem, static_smem, regs);
   return HBT_OK;
@@ -86,11 +93,26 @@ int hbt_occupancy_host_batch(const hbt_device_spec* spec, int64_t n, const int32
                              const int32_t* regs, int32_t* out) {
   if (spec == nullptr || n < 0) return HBT_EINVAL;
   if (n > 0 && (!block_size || !dynamic_smem || !static_smem || !regs || !out)) return HBT_EINVAL;
-  if (spec->warp_size > 32768 || spec->smem_per_block < 0 || spec->smem_per_sm < 0)
-    return HBT_ESPEC;
+  if (!hbt::occupancy_spec_in_domain(*spec)) return HBT_ESPEC;
   const hbt::OccDevice d = hbt::make_occ_device(*spec);
   for (int64_t i = 0; i < n; ++i)
     out[i] = hbt::occupancy_exact(d, block_size[i], dynamic_smem[i], static_smem[i], regs[i]);
+  return HBT_OK;
+}
+
+int hbt_occupancy_host_model32_batch(const hbt_device_spec* spec, int64_t n,
+                                     const int32_t* block_size, const int32_t* dynamic_smem,
+                                     const int32_t* static_smem, const int32_t* regs,
+                                     int32_t* out) {
+  if (spec == nullptr || n < 0) return HBT_EINVAL;
+  if (n > 0 && (!block_size || !dynamic_smem || !static_smem || !regs || !out)) return HBT_EINVAL;
+  if (!hbt::occupancy_spec_in_domain(*spec)) return HBT_ESPEC;
+  const hbt::OccDevice d = hbt::make_occ_device(*spec);
+  if (!d.fast_ok()) return HBT_ESPEC;
+  for (int64_t i = 0; i < n; ++i)
+    out[i] = hbt::occupancy_fast(
+        d, block_size[i], hbt::smem_alloc(hbt::smem_sum(static_smem[i], dynamic_smem[i])),
+        regs[i] & 0xFFFF);
   return HBT_OK;
 }
 
@@ -143,7 +165,7 @@ int hbt_wave_scale(const hbt_device_spec* origin, const hbt_device_spec* dests, 
   a.out_occ_origin = out_occ_origin; a.out_wave_origin = out_wave_origin;
   a.origin = make_occ_device(*origin);
   a.origin_peak_gflops = origin->peak_gflops;
-  a.origin_sms = (double)origin->num_sms;
+  a.origin_inv_sms = 1.0f / (float)origin->num_sms;
 
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
   for (int32_t d0 = 0; d0 < n_dest; d0 += kMaxDestPerLaunch) {

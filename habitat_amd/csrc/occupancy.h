@@ -11,11 +11,14 @@
 // :1165-1282 (registers) and :1289-1420 (combination, GP100 re-check).
 //
 // Layout of the work: everything that depends on the device alone is folded
-// into an OccDevice on the host once per launch; the per-record part is a
-// handful of integer operations and five divisions.  The divisions go through
-// a policy: ExactDiv is plain 64-bit C division (host, and the kernel's rare
-// slow path), FastDiv is a float-reciprocal division that is exact for
-// operands below 2^22 (the kernel's fast path).
+// into an OccDevice on the host once per launch (14 dwords, held in SGPRs by
+// the kernel); the per-record part is a handful of integer operations and
+// three divisions.  Two implementations of that part: occupancy_core in 64-bit
+// arithmetic with plain C division (host, and the kernel variant for devices
+// with huge limits), and occupancy_fast in 32-bit arithmetic with a
+// float-reciprocal division that is exact for operands below 2^22 (the kernel's
+// normal path, taken when every device constant is small enough — which every
+// real device is).
 #pragma once
 
 #include <climits>
@@ -31,40 +34,54 @@
 
 namespace hbt {
 
-enum SmemArch : int32_t { kFixedPool = 0, kVolta = 1, kTuring = 2 };
+// OccDevice::flags
+enum : uint32_t {
+  kOk = 1u << 0,         // the model accepts this device (else occupancy 0 everywhere)
+  kFastOk = 1u << 1,     // every constant is small enough for occupancy_fast
+  kGp100 = 1u << 2,      // cc 6.0: 2 sub-partitions, re-checked with 4
+  kVolta = 1u << 3,      // cc 7.0/7.2: pool steps 0/8/16/32/64 KB/all
+  kTuring = 1u << 4,     // cc 7.5: pool steps 32 KB/all
+  kPoolSteps = 1u << 5,  // cc 7.x and a block's allocation can exceed pref_pool
+  kWarpPow2 = 1u << 6,   // warp_size is a power of two: warp_shift is valid
+};
 
-// Device-only constants of the occupancy model.
+// Device-only constants of the occupancy model.  Every field fits 32 bits:
+// hbt_device_spec_check bounds the shared-memory sizes below 2^31.
 struct OccDevice {
-  int32_t ok;                 // 0: the model rejects this device -> occupancy 0 everywhere
-  int32_t fast_ok;            // 1: every constant below is < 2^22 (FastDiv may be used)
+  uint32_t flags;
   int32_t warp_size;
-  int32_t warp_shift;         // log2(warp_size) when it is a power of two, else -1
+  int32_t warp_shift;         // log2(warp_size) when kWarpPow2
+  int32_t sub_shift;          // log2(sub-partitions): 2, or 1 on cc 6.0
   int32_t max_threads_per_block;
   int32_t max_warps_per_sm;   // max_threads_per_sm / warp_size
   int32_t regs_per_block;
-  int32_t regs_per_subpart;   // regs_per_sm / subparts
+  int32_t regs_per_subpart;   // regs_per_sm / sub-partitions
   int32_t regs_per_subpart4;  // regs_per_sm / 4 (GP100 re-check)
-  int32_t subparts;           // 4, or 2 on cc 6.0
-  int32_t gp100;              // 1 on cc 6.0
   int32_t block_slots;
-  int32_t smem_arch;          // SmemArch
   int32_t num_sms;
-  int64_t smem_per_block;
-  int64_t smem_per_sm;
-  int64_t pref_pool;          // cc 7.x: the pool the default carve-out selects
+  int32_t smem_per_block;
+  int32_t smem_per_sm;
+  int32_t pref_pool;          // cc 7.x: the pool the default carve-out selects
+
+  HBT_HD bool ok() const { return (flags & kOk) != 0; }
+  HBT_HD bool fast_ok() const { return (flags & kFastOk) != 0; }
 };
 
-HBT_HD int64_t volta_pool(int32_t arch, int64_t smem_per_sm, int64_t size) {
-  if (arch == kTuring) return size <= 32768 ? 32768 : smem_per_sm;
-  if (size == 0) return 0;
-  if (size <= 8192) return 8192;
-  if (size <= 16384) return 16384;
-  if (size <= 32768) return 32768;
-  if (size <= 65536) return 65536;
-  return smem_per_sm;
+// Shared-memory pool a cc 7.x SM is configured to for an allocation of `size`
+// (written with selects: `size` differs per lane in the kernel).
+HBT_HD int32_t volta_pool(uint32_t flags, int32_t smem_per_sm, int32_t size) {
+  if (flags & kTuring) return size <= 32768 ? 32768 : smem_per_sm;
+  int32_t p = smem_per_sm;
+  p = size <= 65536 ? 65536 : p;
+  p = size <= 32768 ? 32768 : p;
+  p = size <= 16384 ? 16384 : p;
+  p = size <= 8192 ? 8192 : p;
+  p = size == 0 ? 0 : p;
+  return p;
 }
 
 // Host-side folding of a device spec (cuda_occupancy.h:922-958 for the checks).
+// Expects smem fields in [0, 2^31) and warp_size <= 32768 (callers check).
 inline OccDevice make_occ_device(const hbt_device_spec& s) {
   OccDevice d{};
   const int major = s.compute_major, minor = s.compute_minor;
@@ -72,86 +89,191 @@ inline OccDevice make_occ_device(const hbt_device_spec& s) {
   const bool limits_ok = s.max_threads_per_block > 0 && s.max_threads_per_sm > 0 &&
                          s.regs_per_block > 0 && s.regs_per_sm > 0 && s.warp_size > 0 &&
                          s.smem_per_block != 0 && s.smem_per_sm != 0 && s.num_sms > 0;
-  d.ok = (known && limits_ok) ? 1 : 0;
+  const bool ok = known && limits_ok;
+  const bool gp100 = (major == 6 && minor == 0);
   d.warp_size = s.warp_size > 0 ? s.warp_size : 1;
-  d.warp_shift = -1;
-  if ((d.warp_size & (d.warp_size - 1)) == 0) {
+  const bool pow2 = (d.warp_size & (d.warp_size - 1)) == 0;
+  if (pow2) {
     int sh = 0;
     while ((1 << sh) < d.warp_size) ++sh;
     d.warp_shift = sh;
   }
+  d.sub_shift = gp100 ? 1 : 2;
   d.max_threads_per_block = s.max_threads_per_block;
   d.max_warps_per_sm = s.max_threads_per_sm / d.warp_size;
   d.regs_per_block = s.regs_per_block;
-  d.gp100 = (major == 6 && minor == 0) ? 1 : 0;
-  d.subparts = d.gp100 ? 2 : 4;
-  d.regs_per_subpart = s.regs_per_sm / d.subparts;
+  d.regs_per_subpart = s.regs_per_sm >> d.sub_shift;
   d.regs_per_subpart4 = s.regs_per_sm / 4;
   d.block_slots = (major == 3) ? 16 : (major == 7 && minor == 5) ? 16 : 32;
-  d.smem_arch = (major == 7) ? (minor == 5 ? kTuring : kVolta) : kFixedPool;
   d.num_sms = s.num_sms;
-  d.smem_per_block = s.smem_per_block;
-  d.smem_per_sm = s.smem_per_sm;
-  d.pref_pool = (major == 7) ? volta_pool(d.smem_arch, s.smem_per_sm, s.smem_per_sm)
-                             : s.smem_per_sm;
-  const int64_t lim = (int64_t)1 << 22;
-  d.fast_ok = (d.warp_size < lim && d.max_warps_per_sm < lim && d.regs_per_subpart < lim &&
-               d.smem_per_sm < lim && d.smem_per_sm > 0 && d.pref_pool < lim &&
-               d.smem_per_block > 0)
-                  ? 1 : 0;
+  d.smem_per_block = (int32_t)s.smem_per_block;
+  d.smem_per_sm = (int32_t)s.smem_per_sm;
+  uint32_t flags = 0;
+  if (ok) flags |= kOk;
+  if (gp100) flags |= kGp100;
+  if (major == 7) flags |= (minor == 5) ? kTuring : kVolta;
+  if (pow2) flags |= kWarpPow2;
+  d.pref_pool = (major == 7) ? volta_pool(flags, d.smem_per_sm, d.smem_per_sm) : d.smem_per_sm;
+  if (major == 7 && d.pref_pool < d.smem_per_block) flags |= kPoolSteps;
+  const int32_t lim = 1 << 22;
+  const bool fast = !ok ||  // a rejected device needs no arithmetic at all
+                    (d.warp_size <= 1024 && d.max_threads_per_block < lim - 1024 &&
+                     d.max_warps_per_sm < lim && d.regs_per_subpart < lim &&
+                     d.smem_per_sm < lim && d.pref_pool < lim && d.smem_per_block < lim &&
+                     d.num_sms <= (1 << 14));
+  if (fast) flags |= kFastOk;
+  d.flags = flags;
   return d;
 }
 
-struct ExactDiv {
-  static HBT_HD int64_t div(int64_t a, int64_t b) { return a / b; }
-};
-
-#if defined(__HIPCC__)
-// a / b for 0 <= a < 2^22, 0 < b < 2^22.  float(a), float(b) are exact, the
-// hardware reciprocal is within 1 ulp and the product rounds once more, so the
-// estimate is within 1 of the quotient; one correction step makes it exact.
-struct FastDiv {
-  static __device__ __forceinline__ int64_t div(int64_t a64, int64_t b64) {
-    const int a = (int)a64, b = (int)b64;
-    int q = (int)(__int2float_rn(a) * __builtin_amdgcn_rcpf(__int2float_rn(b)));
-    int r = a - q * b;
-    q += (r >= b) ? 1 : 0;
-    q -= (r < 0) ? 1 : 0;
-    return q;
-  }
-};
+// Exact a / b for 0 <= a < 2^22, 0 < b < 2^24, given rb = 1 / float(b) to within
+// 1 ulp.  float(a) and float(b) are exact and the product rounds once more, so
+// the truncated estimate is within 1 of the quotient; one correction step in
+// each direction makes it exact.  On the host (used to test the 32-bit model)
+// it is plain division.
+HBT_HD float fast_rcp(int32_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_rcpf(__int2float_rn(b));
+#else
+  return 1.0f / (float)b;
 #endif
+}
 
-// The per-record part.  `regs` is already narrowed to 16 bits by the caller.
-// Preconditions for FastDiv: d.fast_ok, block < 2^22, 0 <= static+dyn < 2^22 and
-// regs * warp_size + 255 < 2^22 (callers test these and fall back to ExactDiv).
-template <class Div>
+HBT_HD int32_t fast_div_r(int32_t a, int32_t b, float rb) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  int32_t q = (int32_t)(__int2float_rn(a) * rb);
+  const int32_t r = a - __mul24(q, b);  // q, b < 2^24 and the product fits 32 bits
+  q += (r >= b) ? 1 : 0;
+  q -= (r < 0) ? 1 : 0;
+  return q;
+#else
+  (void)rb;
+  return a / b;
+#endif
+}
+
+HBT_HD int32_t fast_div(int32_t a, int32_t b) { return fast_div_r(a, b, fast_rcp(b)); }
+
+HBT_HD int32_t mul_small(int32_t a, int32_t b) {  // both below 2^23, product below 2^31
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __mul24(a, b);
+#else
+  return a * b;
+#endif
+}
+
+// Wrap-around sum of the two shared-memory sizes: both reach the reference's
+// routine as size_t and the sum is cast to int (cuda_occupancy.h:1101-1102).
+HBT_HD int32_t smem_sum(int32_t static_smem, int32_t dynamic_smem) {
+  return (int32_t)((uint32_t)static_smem + (uint32_t)dynamic_smem);
+}
+
+// The shared-memory allocation of a block: the same on every architecture the
+// model knows (256-byte granularity), so it is computed once per record.
+// The rounding is C division (truncating) and the rounded size is compared as
+// an unsigned 64-bit value: (total + 255) / 256 is 0 for total in -510..0
+// (nothing allocated) and negative, hence enormous, below that.  A sum the
+// 32-bit model cannot hold (enormous, or 2^22 and more) is represented by an
+// allocation of 2^22 bytes, which exceeds the per-block limit of every fast_ok
+// device and so gives occupancy 0 there, as the true value would.
+struct SmemAlloc {
+  int32_t alloc;  // rounded allocation in bytes
+  float rcp;      // 1 / max(alloc, 1)
+};
+
+HBT_HD SmemAlloc smem_alloc(int32_t smem_total) {
+  SmemAlloc s;
+  const bool representable = smem_total >= -510 && smem_total < (1 << 22);
+  const int32_t t = smem_total > 0 ? smem_total : 0;
+  s.alloc = representable ? ((t + 255) & ~255) : (1 << 22);
+  s.rcp = fast_rcp(s.alloc > 0 ? s.alloc : 1);
+  return s;
+}
+
+// The occupancy model in 32-bit arithmetic, for devices with kFastOk (every
+// device constant below 2^22, warp size <= 1024).  Any int32 record is
+// accepted: fields outside the range the divisions are exact for have
+// closed-form answers on such a device.  `regs` is already narrowed to 16 bits.
+//
+// Written without data-dependent branches (a wavefront holds 64 different
+// records): an invalid record keeps computing on clamped operands and its
+// budget is zeroed.  Branches on device constants are wave-uniform.  The
+// register and warp-slot limits share their divisor, and floor division is
+// monotonic, so min(floor(a / w), floor(b / w)) is taken as floor(min(a, b) / w).
+HBT_HD int32_t occupancy_fast(const OccDevice& d, int32_t block, const SmemAlloc& sm,
+                              int32_t regs) {
+  if (!d.ok()) return 0;
+  // regs <= 256 is the per-thread limit; it also keeps regs * warp_size below 2^22
+  const bool in_range = block > 0 && block <= d.max_threads_per_block && regs <= 256;
+  block = in_range ? block : 1;
+  regs = in_range ? regs : 0;
+
+  const int32_t ws = d.warp_size;
+  const int32_t warps = (d.flags & kWarpPow2) ? ((block + ws - 1) >> d.warp_shift)
+                                              : fast_div(block + ws - 1, ws);
+  const float rcp_warps = fast_rcp(warps);
+
+  // registers: 256 per-warp granularity, allocated per sub-partition; a block
+  // must fit the per-block limit with its warps rounded up to the sub-partitions
+  const int32_t per_warp = ((mul_small(regs, ws) + 255) >> 8) << 8;
+  const int32_t sub_mask = (1 << d.sub_shift) - 1;
+  const uint32_t warps_up = (uint32_t)((warps + sub_mask) & ~sub_mask);
+  bool fits = (uint64_t)(uint32_t)per_warp * warps_up <= (uint64_t)(uint32_t)d.regs_per_block;
+  const int32_t per_warp1 = per_warp > 0 ? per_warp : 1;
+  const float rcp_per_warp = fast_rcp(per_warp1);
+  const int32_t reg_warps = fast_div_r(d.regs_per_subpart, per_warp1, rcp_per_warp) << d.sub_shift;
+  if (d.flags & kGp100) {
+    // cc 6.0 must also fit a 4-sub-partition Pascal SM
+    const uint32_t warps_up4 = (uint32_t)((warps + 3) & ~3);
+    fits = fits &&
+           (uint64_t)(uint32_t)per_warp * warps_up4 <= (uint64_t)(uint32_t)d.regs_per_block &&
+           (per_warp == 0 ||
+            (fast_div_r(d.regs_per_subpart4, per_warp1, rcp_per_warp) << 2) >= warps);
+  }
+  int32_t warp_budget = d.max_warps_per_sm;
+  warp_budget = (per_warp > 0 && reg_warps < warp_budget) ? reg_warps : warp_budget;
+  warp_budget = (in_range && fits) ? warp_budget : 0;
+  int32_t lim = fast_div_r(warp_budget, warps, rcp_warps);
+  lim = d.block_slots < lim ? d.block_slots : lim;
+
+  // shared memory: an allocation above the per-block limit leaves no pool
+  int32_t pool = d.pref_pool;
+  if (d.flags & kPoolSteps) {
+    const int32_t stepped = volta_pool(d.flags, d.smem_per_sm, sm.alloc);
+    pool = pool < sm.alloc ? stepped : pool;
+  }
+  pool = sm.alloc <= d.smem_per_block ? pool : 0;
+  const int32_t lim_smem = fast_div_r(pool, sm.alloc > 0 ? sm.alloc : 1, sm.rcp);
+  lim = (sm.alloc > 0 && lim_smem < lim) ? lim_smem : lim;
+  return lim;
+}
+
+// The model without preconditions, in 64-bit arithmetic with C division (host,
+// and the kernel variant for devices outside kFastOk).  `regs` is already
+// narrowed to 16 bits; `smem_total` is smem_sum() of the two sizes.
 HBT_HD int32_t occupancy_core(const OccDevice& d, int32_t block, int32_t smem_total, int32_t regs) {
-  if (!d.ok || block <= 0) return 0;
+  if (!d.ok() || block <= 0) return 0;
   // Block too large: the warp limit is 0 and every limit is >= 0.
   if (block > d.max_threads_per_block) return 0;
 
-  const int64_t warps = (d.warp_shift >= 0)
-                            ? (((int64_t)block + d.warp_size - 1) >> d.warp_shift)
-                            : Div::div((int64_t)block + d.warp_size - 1, d.warp_size);
+  const int64_t warps = ((int64_t)block + d.warp_size - 1) / d.warp_size;
 
   // --- registers -----------------------------------------------------------
   int64_t lim_regs;
   {
     const int64_t per_warp = (((int64_t)regs * d.warp_size + 255) >> 8) << 8;
-    const int64_t sub = d.subparts;
+    const int64_t sub = (int64_t)1 << d.sub_shift;
     const int64_t assumed = per_warp * ((warps + sub - 1) & ~(sub - 1));
     if (d.regs_per_block < assumed || regs > 256) {
       lim_regs = 0;  // `assumed` >= the per-block allocation, one test covers both
     } else if (per_warp == 0) {
       lim_regs = INT_MAX;
     } else {
-      lim_regs = Div::div(Div::div(d.regs_per_subpart, per_warp) * sub, warps);
-      if (d.gp100 && lim_regs != 0) {
+      lim_regs = ((d.regs_per_subpart / per_warp) * sub) / warps;
+      if ((d.flags & kGp100) && lim_regs != 0) {
         // cc 6.0 must also fit a 4-sub-partition Pascal SM.
         const int64_t assumed4 = per_warp * ((warps + 3) & ~(int64_t)3);
-        if (d.regs_per_block < assumed4 ||
-            Div::div(d.regs_per_subpart4, per_warp) * 4 < warps)
+        if (d.regs_per_block < assumed4 || (d.regs_per_subpart4 / per_warp) * 4 < warps)
           lim_regs = 0;
       }
     }
@@ -159,7 +281,7 @@ HBT_HD int32_t occupancy_core(const OccDevice& d, int32_t block, int32_t smem_to
   if (lim_regs == 0) return 0;
 
   // --- warp slots ------------------------------------------------------------
-  const int64_t lim_warps = Div::div(d.max_warps_per_sm, warps);
+  const int64_t lim_warps = d.max_warps_per_sm / warps;
 
   // --- shared memory ---------------------------------------------------------
   int64_t lim_smem;
@@ -173,9 +295,9 @@ HBT_HD int32_t occupancy_core(const OccDevice& d, int32_t block, int32_t smem_to
       lim_smem = INT_MAX;
     } else {
       int64_t pool = d.pref_pool;
-      if (d.smem_arch != kFixedPool && pool < alloc)
-        pool = volta_pool(d.smem_arch, d.smem_per_sm, alloc);
-      lim_smem = (int32_t)Div::div(pool, alloc);
+      if ((d.flags & (kVolta | kTuring)) && pool < alloc)
+        pool = volta_pool(d.flags, d.smem_per_sm, (int32_t)alloc);  // alloc <= smem_per_block < 2^31
+      lim_smem = (int32_t)(pool / alloc);
     }
   }
 
@@ -186,17 +308,10 @@ HBT_HD int32_t occupancy_core(const OccDevice& d, int32_t block, int32_t smem_to
   return (int32_t)m;
 }
 
-// Wrap-around sum of the two shared-memory sizes: both reach the reference's
-// routine as size_t and the sum is cast to int (cuda_occupancy.h:1101-1102).
-HBT_HD int32_t smem_sum(int32_t static_smem, int32_t dynamic_smem) {
-  return (int32_t)((uint32_t)static_smem + (uint32_t)dynamic_smem);
-}
-
 // Host / slow-path occupancy: no preconditions.
 HBT_HD int32_t occupancy_exact(const OccDevice& d, int32_t block, int32_t dynamic_smem,
                                int32_t static_smem, int32_t regs) {
-  return occupancy_core<ExactDiv>(d, block, smem_sum(static_smem, dynamic_smem),
-                                  (int32_t)(uint16_t)regs);
+  return occupancy_core(d, block, smem_sum(static_smem, dynamic_smem), (int32_t)(uint16_t)regs);
 }
 
 }  // namespace hbt

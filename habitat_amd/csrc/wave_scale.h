@@ -17,14 +17,14 @@ constexpr int kMaxDestPerLaunch = 8;
 // (analyzer/habitat/analysis/wave_scaling/roofline.py:48-64, :107-108).
 struct DestArgs {
   OccDevice dev;
-  double sms;                  // num_sms as a double
   double ridge;                // peak_gflops / mem_bandwidth_gb
   double half_ridge;           // 0.5 * ridge
   double neg_half_over_ridge;  // -0.5 / ridge
   double bw_ratio;             // origin.mem_bandwidth_gb / dest.mem_bandwidth_gb
-  double clk_ratio;            // origin.base_clock_mhz / dest.base_clock_mhz
   double log2_bw;              // log2(bw_ratio)
-  double log2_clk_sm;          // log2(clk_ratio) + log2(origin.num_sms / dest.num_sms)
+  double log2_clk;             // log2(origin.base_clock_mhz / dest.base_clock_mhz)
+  double log2_clk_sm;          // log2_clk + log2(origin.num_sms / dest.num_sms)
+  float inv_sms;               // 1 / num_sms rounded to float
 };
 
 struct WaveScaleArgs {
@@ -50,7 +50,7 @@ struct WaveScaleArgs {
   uint8_t* out_status;         // [n_dest][n], nullable
   OccDevice origin;
   double origin_peak_gflops;
-  double origin_sms;
+  float origin_inv_sms;        // 1 / origin.num_sms rounded to float
   DestArgs dest[kMaxDestPerLaunch];
 };
 

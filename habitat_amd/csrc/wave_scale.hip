@@ -28,8 +28,24 @@ namespace hbt {
 
 namespace {
 
-constexpr int kRecPerThread = 4;
+constexpr int kRecPerThread = 2;
 constexpr int kBlock = 256;
+
+// log2(i) for i = 0..32 (entry 0 unused), padded to one entry per lane.  A
+// kernel that fits in one wave on a device has num_blocks < num_sms * occupancy
+// with occupancy <= 32 block slots, so ceil(num_blocks / num_sms) is an integer
+// in 1..32 and the logarithm of the small-kernel factor needs no more than this
+// table.  Each wavefront keeps it in one register pair (lane i holds entry i)
+// and looks entries up with a cross-lane permute: no LDS, no barrier.
+__device__ const double kLog2Int[64] = {
+    0x0.0p+0, 0x0.0p+0, 0x1.0000000000000p+0, 0x1.95c01a39fbd68p+0, 0x1.0000000000000p+1,
+    0x1.2934f0979a371p+1, 0x1.4ae00d1cfdeb4p+1, 0x1.675767f54042dp+1, 0x1.8000000000000p+1,
+    0x1.95c01a39fbd68p+1, 0x1.a934f0979a371p+1, 0x1.bacea7c065d42p+1, 0x1.cae00d1cfdeb4p+1,
+    0x1.d9a802391e233p+1, 0x1.e75767f54042dp+1, 0x1.f414fdb498226p+1, 0x1.0000000000000p+2,
+    0x1.0598fdbeb244cp+2, 0x1.0ae00d1cfdeb4p+2, 0x1.0fde0b5c81340p+2, 0x1.149a784bcd1b9p+2,
+    0x1.191bba891f171p+2, 0x1.1d6753e032ea1p+2, 0x1.21820a01ac755p+2, 0x1.2570068e7ef5ap+2,
+    0x1.2934f0979a371p+2, 0x1.2cd4011c8f119p+2, 0x1.305013ab7ce0ep+2, 0x1.33abb3faa0216p+2,
+    0x1.36e9291eaa65bp+2, 0x1.3a0a7eda4c113p+2, 0x1.3d118d66c4d4ep+2, 0x1.4000000000000p+2};
 
 struct RecordIn {
   int32_t nb, block, smem_total, regs, dest_regs;
@@ -39,33 +55,92 @@ struct RecordIn {
 
 // Destination-independent part of one record.
 struct RecordMid {
+  SmemAlloc smem;
   int32_t occ_o, wave_o;
-  bool small_o;       // num_blocks // origin_wave == 0
-  bool fast;          // operands small enough for the float-reciprocal division
-  double num_gflops, total_gb, intensity;
-  double origin_max_occ;  // ceil(num_blocks / origin.num_sms)
+  int32_t origin_max_occ;  // ceil(num_blocks / origin.num_sms) when small_o, else 0
+  bool small_o;            // num_blocks // origin_wave == 0
+  double num_gflops, total_gb;
 };
 
-__device__ __forceinline__ int32_t occupancy_dev(const OccDevice& d, bool fast, int32_t block,
-                                                 int32_t smem_total, int32_t regs) {
-  regs &= 0xFFFF;  // uint16_t narrowing, cpp/src/cuda/kernel.h:108
-  if (fast && d.fast_ok && (int64_t)regs * d.warp_size + 255 < (1 << 22))
-    return occupancy_core<FastDiv>(d, block, smem_total, regs);
-  return occupancy_core<ExactDiv>(d, block, smem_total, regs);
+// 2^x for finite x, relative error below 1e-13: split x = n + f with
+// |f| <= 1/2, evaluate e^(f ln 2) by its Taylor polynomial of degree 11
+// ((ln2 / 2)^12 / 12! < 7e-15) and scale by 2^n.
+__device__ __forceinline__ double exp2_poly(double x) {
+  const double n = rint(x);
+  const double z = (x - n) * 0x1.62e42fefa39efp-1;  // f * ln 2
+  double p = 1.0 / 39916800.0;
+  p = fma(p, z, 1.0 / 3628800.0);
+  p = fma(p, z, 1.0 / 362880.0);
+  p = fma(p, z, 1.0 / 40320.0);
+  p = fma(p, z, 1.0 / 5040.0);
+  p = fma(p, z, 1.0 / 720.0);
+  p = fma(p, z, 1.0 / 120.0);
+  p = fma(p, z, 1.0 / 24.0);
+  p = fma(p, z, 1.0 / 6.0);
+  p = fma(p, z, 0.5);
+  p = fma(p, z, 1.0);
+  p = fma(p, z, 1.0);
+  // |x| beyond the exponent range saturates through ldexp (inf or 0)
+  const double nc = fmin(fmax(n, -4096.0), 4096.0);
+  return ldexp(p, (int)nc);
 }
 
+// x / c for a compile-time constant c, correctly rounded like the IEEE
+// division it replaces: q = x * (1/c) is within an ulp of the quotient, the
+// remainder x - q*c is exact in an FMA, and adding remainder * (1/c) back
+// rounds to the nearest double (Markstein's correction; checked against `/`
+// on 4e8 operands for each constant used here).  Operands whose remainder
+// could underflow or overflow take the hardware sequence instead.
+template <class C>
+__device__ __forceinline__ double div_const(double x) {
+  constexpr double c = C::value, rc = 1.0 / C::value;
+  const double ax = fabs(x);
+  if (__builtin_expect((ax > 0x1p+900) || (ax < 0x1p-900 && ax != 0.0), 0)) return x / c;
+  const double q = x * rc;
+  const double r = fma(-q, c, x);
+  return fma(r, rc, q);
+}
+struct C100 { static constexpr double value = 100.0; };
+struct C1e9 { static constexpr double value = 1e9; };
+
+// FAST: every device of the launch has OccDevice::fast_ok, so the 32-bit model
+// applies to every record.  Otherwise the 64-bit model with real divisions runs
+// (devices with limits of 2^22 and more: not real hardware, but in the domain).
+template <bool FAST>
+__device__ __forceinline__ int32_t occupancy_dev(const OccDevice& d, int32_t block,
+                                                 int32_t smem_total, const SmemAlloc& sm,
+                                                 int32_t regs) {
+  regs &= 0xFFFF;  // uint16_t narrowing, cpp/src/cuda/kernel.h:108
+  if (FAST) return occupancy_fast(d, block, sm, regs);
+  return occupancy_core(d, block, smem_total, regs);
+}
+
+// ceil(nb / sms) for 0 <= nb < 32 * sms.  The reference takes math.ceil of the
+// fp64 quotient (roofline.py:33-38); for operands below 2^53 that quotient is an
+// integer only when the division is exact, so the integer ceiling is the same.
+// On a fast_ok device sms <= 2^14 and nb < 2^19: float(nb) * (1/sms) is within
+// 2^-18 of the quotient, which is either an integer or at least 2^-14 away from
+// one, so ceil(product - 2^-16) is the exact ceiling.
+template <bool FAST>
+__device__ __forceinline__ int32_t ceil_div_small(int32_t nb, int32_t sms, float inv_sms) {
+  if (FAST) return (int32_t)ceilf(fmaf(__int2float_rn(nb), inv_sms, -0x1p-16f));
+  return (int32_t)(((int64_t)nb + sms - 1) / sms);
+}
+
+template <bool FAST>
 __device__ __forceinline__ RecordMid origin_part(const WaveScaleArgs& a, const RecordIn& r) {
   RecordMid m;
-  m.fast = r.block < (1 << 22) && r.smem_total >= 0 && r.smem_total < (1 << 22);
-  m.occ_o = occupancy_dev(a.origin, m.fast, r.block, r.smem_total, r.regs);
-  m.wave_o = a.origin.num_sms * m.occ_o;
+  m.smem = smem_alloc(r.smem_total);
+  m.occ_o = occupancy_dev<FAST>(a.origin, r.block, r.smem_total, m.smem, r.regs);
+  m.wave_o = mul_small(a.origin.num_sms, m.occ_o);
   m.small_o = r.nb >= 0 && r.nb < m.wave_o;
-  // roofline.py:72-76, same operation order
+  m.origin_max_occ =
+      ceil_div_small<FAST>(m.small_o ? r.nb : 0, a.origin.num_sms, a.origin_inv_sms);
+  // roofline.py:72-76, same operation order (the three divisions by 1024 are
+  // exact scalings)
   m.total_gb = (r.rd + r.wr) / 1024 / 1024 / 1024;
-  const double gflops_per_second = r.eff / 100 * a.origin_peak_gflops;
-  m.num_gflops = gflops_per_second * r.t / 1e9;
-  m.intensity = m.num_gflops / m.total_gb;
-  m.origin_max_occ = ceil((double)r.nb / a.origin_sms);
+  const double gflops_per_second = div_const<C100>(r.eff) * a.origin_peak_gflops;
+  m.num_gflops = div_const<C1e9>(gflops_per_second * r.t);
   return m;
 }
 
@@ -75,106 +150,110 @@ struct RecordOut {
   uint8_t status;
 };
 
+// Written with selects rather than branches: the 64 records of a wavefront
+// take all paths between them anyway.
+// log2 of a small-kernel block count (0..32).  PERMUTE: read it from the lane
+// that holds it (needs all 64 lanes of the wavefront active); otherwise gather
+// it from the table in memory.
+template <bool PERMUTE>
+__device__ __forceinline__ double log2_count(double log2_lane, int32_t count) {
+  if (PERMUTE) return __shfl(log2_lane, count & 63);
+  return kLog2Int[count & 63];
+}
+
+template <bool FAST, bool PERMUTE>
 __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn& r,
-                                               const RecordMid& m) {
+                                               const RecordMid& m, double log2_lane) {
   RecordOut o;
   const int32_t regs_d = r.dest_regs >= 0 ? r.dest_regs : r.regs;
-  o.occ_d = occupancy_dev(p.dev, m.fast, r.block, r.smem_total, regs_d);
-  o.wave_d = p.dev.num_sms * o.occ_d;
-  o.t = __builtin_nan("");
+  o.occ_d = occupancy_dev<FAST>(p.dev, r.block, r.smem_total, m.smem, regs_d);
+  o.wave_d = mul_small(p.dev.num_sms, o.occ_d);
 
-  double gamma = 1.0;
-  if (r.metrics) {
-    // roofline.py:86-101
-    if (m.num_gflops < 1e-9) gamma = 1.;
-    else if (m.total_gb == 0) gamma = 0.;
-    else if (m.intensity > p.ridge) gamma = p.half_ridge / m.intensity;
-    else gamma = p.neg_half_over_ridge * m.intensity + 1.;
-    if (!(gamma >= 0 && gamma <= 1)) { o.status = HBT_ST_BAD_GAMMA; return o; }
-  }
-  if (m.wave_o == 0) { o.status = HBT_ST_ORIGIN_WAVE_ZERO; return o; }
-  bool small = m.small_o;
-  if (small) {
-    if (o.wave_d == 0) { o.status = HBT_ST_DEST_WAVE_ZERO; return o; }
-    small = r.nb < o.wave_d;
-  }
-  o.status = HBT_ST_OK;
+  // roofline.py:86-101.  With I = gflops / gb the reference takes
+  // 0.5 * R / I above the ridge point R and 1 - 0.5 / R * I below; both are
+  // formed here from one division by choosing its operands first.  The choice
+  // compares gflops with R * gb instead of I with R, which can differ only
+  // within an ulp of the ridge, where the two expressions agree (gamma = 1/2).
+  const bool above = m.total_gb > 0 && m.num_gflops > p.ridge * m.total_gb;
+  const double q = (above ? p.half_ridge * m.total_gb : m.num_gflops) /
+                   (above ? m.num_gflops : m.total_gb);
+  double gamma = above ? q : p.neg_half_over_ridge * q + 1.;
+  gamma = (m.total_gb == 0) ? 0. : gamma;
+  gamma = (m.num_gflops < 1e-9) ? 1. : gamma;
+  const bool bad_gamma = r.metrics && !(gamma >= 0 && gamma <= 1);
 
-  if (!r.metrics) {  // resimplified.py:25-40
-    o.t = small ? r.t : r.t * p.bw_ratio;
-    return o;
-  }
+  // `a // wave_o == 0 and a // wave_d == 0`: the second test, and its division
+  // by zero, happen only when the first holds (roofline.py:29-30).
+  const bool small = m.small_o && r.nb < o.wave_d;
+  const int32_t dest_max_occ = ceil_div_small<FAST>(small ? r.nb : 0, p.dev.num_sms, p.inv_sms);
+
+  int32_t status = HBT_ST_OK;
+  status = (r.metrics && small && m.origin_max_occ == 0) ? HBT_ST_ZERO_BLOCKS : status;
+  status = (m.small_o && o.wave_d == 0) ? HBT_ST_DEST_WAVE_ZERO : status;
+  status = (m.wave_o == 0) ? HBT_ST_ORIGIN_WAVE_ZERO : status;
+  status = bad_gamma ? HBT_ST_BAD_GAMMA : status;
+  o.status = (uint8_t)status;
+
+  // roofline.py:32-45: (clk_ratio * dest_max_occ / origin_max_occ)^(1-gamma), both
+  // counts in 1..32; roofline.py:48-64: bw^gamma * clk^(1-gamma) * sm^(1-gamma)
   const double gamma_compl = 1.0 - gamma;
-  if (small) {       // roofline.py:32-45
-    if (m.origin_max_occ == 0) { o.status = HBT_ST_ZERO_BLOCKS; return o; }
-    const double dest_max_occ = ceil((double)r.nb / p.sms);
-    const double factor = p.clk_ratio * (dest_max_occ / m.origin_max_occ);
-    o.t = r.t * exp2(gamma_compl * log2(factor));
-    return o;
-  }
-  // roofline.py:48-64: t * bw^gamma * clk^(1-gamma) * sm^(1-gamma), with the
-  // three logarithms taken once on the host.
-  o.t = r.t * exp2(gamma * p.log2_bw + gamma_compl * p.log2_clk_sm);
+  const double log2_small =
+      p.log2_clk + log2_count<PERMUTE>(log2_lane, dest_max_occ) -
+      log2_count<PERMUTE>(log2_lane, m.origin_max_occ);
+  const double exponent =
+      small ? gamma_compl * log2_small : gamma * p.log2_bw + gamma_compl * p.log2_clk_sm;
+  const double t_roofline = r.t * exp2_poly(exponent);
+  // resimplified.py:25-40
+  const double t_plain = small ? r.t : r.t * p.bw_ratio;
+  const double t = r.metrics ? t_roofline : t_plain;
+  o.t = (status == HBT_ST_OK) ? t : __builtin_nan("");
   return o;
 }
 
 template <class T, int N>
 struct alignas(sizeof(T) * N) Pack { T v[N]; };
 
-// Load R consecutive elements starting at i (vectorised when all are in range).
+// R consecutive elements starting at i, all in range: one vector access.
 template <class T, int R>
-__device__ __forceinline__ void load_r(const T* __restrict__ p, int64_t i, int64_t n, T fill,
-                                       T (&out)[R]) {
-  if (R > 1 && i + R <= n) {
-    const Pack<T, R> v = *reinterpret_cast<const Pack<T, R>*>(p + i);
+__device__ __forceinline__ void load_r(const T* __restrict__ p, int64_t i, T (&out)[R]) {
+  const Pack<T, R> v = *reinterpret_cast<const Pack<T, R>*>(p + i);
 #pragma unroll
-    for (int k = 0; k < R; ++k) out[k] = v.v[k];
-  } else {
-#pragma unroll
-    for (int k = 0; k < R; ++k) out[k] = (i + k < n) ? p[i + k] : fill;
-  }
+  for (int k = 0; k < R; ++k) out[k] = v.v[k];
 }
 
 template <class T, int R>
-__device__ __forceinline__ void store_r(T* __restrict__ p, int64_t i, int64_t n, const T (&in)[R]) {
-  if (R > 1 && i + R <= n) {
-    Pack<T, R> v;
+__device__ __forceinline__ void store_r(T* __restrict__ p, int64_t i, const T (&in)[R]) {
+  Pack<T, R> v;
 #pragma unroll
-    for (int k = 0; k < R; ++k) v.v[k] = in[k];
-    *reinterpret_cast<Pack<T, R>*>(p + i) = v;
-  } else {
-#pragma unroll
-    for (int k = 0; k < R; ++k)
-      if (i + k < n) p[i + k] = in[k];
-  }
+  for (int k = 0; k < R; ++k) v.v[k] = in[k];
+  *reinterpret_cast<Pack<T, R>*>(p + i) = v;
 }
 
-template <int R>
-__global__ __launch_bounds__(kBlock) void wave_scale_kernel(const WaveScaleArgs a) {
-  const int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * R;
-  if (i >= a.n) return;
+// Records i .. i+R-1 (all below n) for every destination of the launch.
+template <int R, bool FAST, bool PERMUTE>
+__device__ __forceinline__ void process(const WaveScaleArgs& a, int64_t i) {
   const int64_t n = a.n;
-
+  const double log2_lane = PERMUTE ? kLog2Int[threadIdx.x & 63] : 0.0;
   int32_t nb[R], block[R], dyn[R], stat[R], regs[R], dregs[R];
   uint8_t hm[R];
   double t[R], eff[R], rd[R], wr[R];
-  load_r<int32_t, R>(a.num_blocks, i, n, 1, nb);
-  load_r<int32_t, R>(a.block_size, i, n, 1, block);
-  load_r<int32_t, R>(a.dynamic_smem, i, n, 0, dyn);
-  load_r<int32_t, R>(a.static_smem, i, n, 0, stat);
-  load_r<int32_t, R>(a.regs, i, n, 0, regs);
-  load_r<double, R>(a.run_time_ns, i, n, 0.0, t);
-  load_r<double, R>(a.flop_sp_efficiency, i, n, 0.0, eff);
-  load_r<double, R>(a.dram_read_bytes, i, n, 0.0, rd);
-  load_r<double, R>(a.dram_write_bytes, i, n, 0.0, wr);
+  load_r<int32_t, R>(a.num_blocks, i, nb);
+  load_r<int32_t, R>(a.block_size, i, block);
+  load_r<int32_t, R>(a.dynamic_smem, i, dyn);
+  load_r<int32_t, R>(a.static_smem, i, stat);
+  load_r<int32_t, R>(a.regs, i, regs);
+  load_r<double, R>(a.run_time_ns, i, t);
+  load_r<double, R>(a.flop_sp_efficiency, i, eff);
+  load_r<double, R>(a.dram_read_bytes, i, rd);
+  load_r<double, R>(a.dram_write_bytes, i, wr);
   if (a.dest_regs != nullptr) {
-    load_r<int32_t, R>(a.dest_regs, i, n, -1, dregs);
+    load_r<int32_t, R>(a.dest_regs, i, dregs);
   } else {
 #pragma unroll
     for (int k = 0; k < R; ++k) dregs[k] = -1;
   }
   if (a.has_metrics != nullptr) {
-    load_r<uint8_t, R>(a.has_metrics, i, n, 1, hm);
+    load_r<uint8_t, R>(a.has_metrics, i, hm);
   } else {
 #pragma unroll
     for (int k = 0; k < R; ++k) hm[k] = 1;
@@ -186,48 +265,71 @@ __global__ __launch_bounds__(kBlock) void wave_scale_kernel(const WaveScaleArgs 
   for (int k = 0; k < R; ++k) {
     rin[k] = RecordIn{nb[k], block[k], smem_sum(stat[k], dyn[k]), regs[k], dregs[k],
                       hm[k] != 0, t[k], eff[k], rd[k], wr[k]};
-    mid[k] = origin_part(a, rin[k]);
+    mid[k] = origin_part<FAST>(a, rin[k]);
   }
 
   if (a.write_origin) {
     int32_t occ_o[R], wave_o[R];
 #pragma unroll
     for (int k = 0; k < R; ++k) { occ_o[k] = mid[k].occ_o; wave_o[k] = mid[k].wave_o; }
-    if (a.out_occ_origin != nullptr) store_r<int32_t, R>(a.out_occ_origin, i, n, occ_o);
-    if (a.out_wave_origin != nullptr) store_r<int32_t, R>(a.out_wave_origin, i, n, wave_o);
+    if (a.out_occ_origin != nullptr) store_r<int32_t, R>(a.out_occ_origin, i, occ_o);
+    if (a.out_wave_origin != nullptr) store_r<int32_t, R>(a.out_wave_origin, i, wave_o);
   }
 
   for (int d = 0; d < a.n_dest; ++d) {
     const DestArgs& p = a.dest[d];
-    const int64_t row = (int64_t)d * n;
+    const int64_t at = (int64_t)d * n + i;
     double ot[R];
     int32_t occ_d[R], wave_d[R];
     uint8_t st[R];
 #pragma unroll
     for (int k = 0; k < R; ++k) {
-      const RecordOut o = dest_part(p, rin[k], mid[k]);
+      const RecordOut o = dest_part<FAST, PERMUTE>(p, rin[k], mid[k], log2_lane);
       ot[k] = o.t; occ_d[k] = o.occ_d; wave_d[k] = o.wave_d; st[k] = o.status;
     }
-    store_r<double, R>(a.out_time_ns + row, i, n, ot);
-    if (a.out_occ_dest != nullptr) store_r<int32_t, R>(a.out_occ_dest + row, i, n, occ_d);
-    if (a.out_wave_dest != nullptr) store_r<int32_t, R>(a.out_wave_dest + row, i, n, wave_d);
-    if (a.out_status != nullptr) store_r<uint8_t, R>(a.out_status + row, i, n, st);
+    store_r<double, R>(a.out_time_ns, at, ot);
+    if (a.out_occ_dest != nullptr) store_r<int32_t, R>(a.out_occ_dest, at, occ_d);
+    if (a.out_wave_dest != nullptr) store_r<int32_t, R>(a.out_wave_dest, at, wave_d);
+    if (a.out_status != nullptr) store_r<uint8_t, R>(a.out_status, at, st);
   }
+}
+
+template <int R, bool FAST>
+__global__ __launch_bounds__(kBlock) void wave_scale_kernel(const WaveScaleArgs a) {
+  const int64_t thread = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t i = thread * R;
+  // A wavefront whose 64 * R records are all in range takes the vector path
+  // with every lane active; the last, partial wavefront of the batch goes one
+  // record at a time.
+  const int64_t wave_end = ((thread | 63) + 1) * R;
+  if (wave_end <= a.n) {
+    process<R, FAST, true>(a, i);
+  } else {
+    const int64_t end = (i + R < a.n) ? i + R : a.n;
+    for (int64_t j = i; j < end; ++j) process<1, FAST, false>(a, j);
+  }
+}
+
+template <int R, bool FAST>
+void launch(const WaveScaleArgs& args, hipStream_t stream) {
+  const int64_t threads = (args.n + R - 1) / R;
+  const int64_t blocks = (threads + kBlock - 1) / kBlock;
+  hipLaunchKernelGGL((wave_scale_kernel<R, FAST>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,
+                     args);
 }
 
 }  // namespace
 
 hipError_t launch_wave_scale(const WaveScaleArgs& args, bool vectorised, hipStream_t stream) {
   if (args.n <= 0) return hipSuccess;
+  bool fast = args.origin.fast_ok();
+  for (int d = 0; d < args.n_dest; ++d) fast = fast && args.dest[d].dev.fast_ok();
   if (vectorised) {
-    const int64_t threads = (args.n + kRecPerThread - 1) / kRecPerThread;
-    const int64_t blocks = (threads + kBlock - 1) / kBlock;
-    hipLaunchKernelGGL(wave_scale_kernel<kRecPerThread>, dim3((unsigned)blocks), dim3(kBlock), 0,
-                       stream, args);
+    if (fast) launch<kRecPerThread, true>(args, stream);
+    else launch<kRecPerThread, false>(args, stream);
   } else {
-    const int64_t blocks = (args.n + kBlock - 1) / kBlock;
-    hipLaunchKernelGGL(wave_scale_kernel<1>, dim3((unsigned)blocks), dim3(kBlock), 0, stream,
-                       args);
+    if (fast) launch<1, true>(args, stream);
+    else launch<1, false>(args, stream);
   }
   return hipGetLastError();
 }

@@ -29,15 +29,17 @@ def _draw_records(rng, n):
     return rec
 
 
-def host_occupancy(device, rec):
-    """Occupancy of every record on `device` (host loop inside the library)."""
+def host_occupancy(device, rec, model32=False):
+    """Occupancy of every record on `device` (host loop inside the library).
+    `model32` evaluates the kernel's 32-bit formulation instead."""
     n = rec["block_size"].shape[0]
     out = np.empty(n, np.int32)
     p = lambda a: a.ctypes.data_as(ctypes.c_void_p)
     cols = [np.ascontiguousarray(rec[k], np.int32)
             for k in ("block_size", "dynamic_smem", "static_smem", "regs_per_thread")]
-    rc = _lib.lib().hbt_occupancy_host_batch(ctypes.byref(device.spec), n, *[p(c) for c in cols],
-                                             p(out))
+    fn = (_lib.lib().hbt_occupancy_host_model32_batch if model32
+          else _lib.lib().hbt_occupancy_host_batch)
+    rc = fn(ctypes.byref(device.spec), n, *[p(c) for c in cols], p(out))
     _lib.check(rc, "hbt_occupancy_host_batch")
     return out
 

@@ -93,6 +93,19 @@ int hbt_occupancy_host_batch(const hbt_device_spec *spec, int64_t n, const int32
                              const int32_t *regs, int32_t *out);
 
 /*
+ * Diagnostic: the 32-bit formulation of the same model that the wave-scaling
+ * kernel uses for devices whose limits are all below 2^22, evaluated on the
+ * HOST over host arrays (its float-reciprocal divisions replaced by exact
+ * ones).  Lets the kernel's integer logic be checked against
+ * hbt_occupancy_host_batch without a GPU.  Returns HBT_ESPEC for a device
+ * outside that formulation's domain.  No counterpart in the reference.
+ */
+int hbt_occupancy_host_model32_batch(const hbt_device_spec *spec, int64_t n,
+                                     const int32_t *block_size, const int32_t *dynamic_smem,
+                                     const int32_t *static_smem, const int32_t *regs,
+                                     int32_t *out);
+
+/*
  * Wave-scale n kernel records measured on `origin` to each of n_dest
  * destination devices.  One launch replaces the per-kernel Python loop of
  * Predictor._wave_scale (analyzer/habitat/analysis/predictor.py:116-124) and,

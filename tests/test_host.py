@@ -59,6 +59,41 @@ def test_host_occupancy_matches_reference_golden(occupancy_golden):
                                               int(g["regs"][i])) == g["occ_own__" + name][i]
 
 
+def test_kernel_32bit_occupancy_model_matches_reference_golden(occupancy_golden):
+    """The formulation the HIP kernel runs (32-bit, closed forms for out-of-range
+    fields), evaluated on the host, against the reference-compiled fixture and
+    against random int32 garbage through the 64-bit host routine."""
+    g, devices = occupancy_golden
+    regs = np.where(g["dregs"] >= 0, g["dregs"], g["regs"]).astype(np.int32)
+    rec = dict(block_size=g["block"], dynamic_smem=g["dyn"], static_smem=g["stat"],
+               regs_per_thread=regs)
+    rng = np.random.default_rng(17)
+    n = 200_000
+    wild = dict(block_size=rng.integers(-5, 3000, n).astype(np.int32),
+                dynamic_smem=rng.integers(-70000, 200000, n).astype(np.int32),
+                static_smem=rng.integers(-70000, 70000, n).astype(np.int32),
+                regs_per_thread=rng.integers(0, 70000, n).astype(np.int32))
+    wild["dynamic_smem"][::7] = rng.integers(-2**31, 2**31 - 1, wild["dynamic_smem"][::7].shape[0])
+    wild["regs_per_thread"][::3] = rng.integers(0, 300, wild["regs_per_thread"][::3].shape[0])
+    wild["dynamic_smem"][::2] = rng.integers(0, 50000, wild["dynamic_smem"][::2].shape[0])
+    wild["static_smem"][::2] = 0
+    # keep clear of the reference's signed overflow: (int)(static + dyn) + 255
+    tot = ((wild["static_smem"].astype(np.int64) + wild["dynamic_smem"] + 2**31) % 2**32) - 2**31
+    keep = tot <= 2**31 - 1 - 255
+    wild = {k: v[keep] for k, v in wild.items()}
+    for name, props in devices.items():
+        dev = DeviceProperties(name=name, **props)
+        assert np.array_equal(synthetic.host_occupancy(dev, rec, model32=True),
+                              g["occ_lut__" + name]), name
+        a = synthetic.host_occupancy(dev, wild, model32=True)
+        b = synthetic.host_occupancy(dev, wild)
+        assert np.array_equal(a, b), name
+        assert name in ("A100like_cc80", "zero_optin_smem_block0") or (a > 0).mean() > 0.01
+    huge = DeviceProperties(name="huge", **dict(Device.V100.as_dict(), regs_per_multiprocessor=1 << 30))
+    with pytest.raises(_lib.HabitatLibraryError):
+        synthetic.host_occupancy(huge, rec, model32=True)
+
+
 def test_kernel_instance_occupancy_known_answers(kat):
     from habitat_amd.analysis.kernels import KernelInstance
     for dev, block, regs, stat, dyn, occ, _ in kat["occupancy"]:
