@@ -44,14 +44,14 @@ using f32x16 = float __attribute__((ext_vector_type(16)));
 constexpr int kWidth = 1024;      // hidden width the kernel is built for
 constexpr int kRows = 32;         // rows per workgroup (one MFMA tile of m)
 constexpr int kStride = kWidth + 4;  // LDS row stride in floats
-constexpr int kMaxInPadded = 64;  // in_features padded to a multiple of 16, at most this
+constexpr int kMaxInPadded = 64;  // in_features padded to a multiple of 32, at most this
 
 struct MlpArgs {
   const double* raw;     // [n][in_features]
   float* out;            // [n]
   int64_t n;
   int32_t in_features;
-  int32_t in_padded;     // multiple of 16
+  int32_t in_padded;     // multiple of 32
   int32_t hidden;
   const double* mu;      // [in_features]
   const double* sigma;   // [in_features]
@@ -62,45 +62,62 @@ struct MlpArgs {
   float b_last;
 };
 
-// One layer's K loop for this wave: acc[tile] += Wfrag * Actfrag over kg groups of 8 k.
+// One layer's K loop for this wave: acc[tile] += Wfrag * Actfrag over kg groups
+// of 8 k (kg a multiple of 4).  Fragments travel through a ring of four
+// register slots: the loads for group j+3 are issued before the MFMAs of group
+// j, so a fragment has three MFMA blocks (>= 3 * 16 * TPW * 4 cycles) to arrive.
+template <int TPW>
+struct Ring {
+  f32x4 w[4][TPW];
+  f32x4 x[4];
+};
+
+template <int TPW, int SLOT>
+__device__ __forceinline__ void ring_load(Ring<TPW>& r, const f32x4* __restrict__ wp, int g,
+                                          const float* act_lane, int lane) {
+  const f32x4* p = wp + (size_t)g * TPW * 64 + lane;
+#pragma unroll
+  for (int t = 0; t < TPW; ++t) r.w[SLOT][t] = p[t * 64];
+  r.x[SLOT] = *reinterpret_cast<const f32x4*>(act_lane + 8 * g);
+}
+
+template <int TPW, int SLOT>
+__device__ __forceinline__ void ring_mfma(const Ring<TPW>& r, f32x16 (&acc)[TPW]) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+      acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(r.w[SLOT][t][e], r.x[SLOT][e], acc[t], 0, 0, 0);
+}
+
 template <int TPW>
 __device__ __forceinline__ void layer_k_loop(const f32x4* __restrict__ wp, int kg,
                                              const float* act_lane, f32x16 (&acc)[TPW]) {
   const int lane = threadIdx.x & 63;
-  f32x4 wa[TPW], wb[TPW];
-  f32x4 xa, xb;
-#pragma unroll
-  for (int t = 0; t < TPW; ++t) wa[t] = wp[t * 64 + lane];
-  xa = *reinterpret_cast<const f32x4*>(act_lane);
-  for (int j = 0; j < kg; j += 2) {
-    // The scheduling barriers keep the compiler from sinking the prefetches
-    // below the MFMA block they are meant to overlap with.
-    {
-      const f32x4* p = wp + (size_t)(j + 1) * TPW * 64 + lane;
-#pragma unroll
-      for (int t = 0; t < TPW; ++t) wb[t] = p[t * 64];
-      xb = *reinterpret_cast<const f32x4*>(act_lane + 8 * (j + 1));
-    }
+  const int last = kg - 1;
+  Ring<TPW> r;
+  ring_load<TPW, 0>(r, wp, 0, act_lane, lane);
+  ring_load<TPW, 1>(r, wp, 1, act_lane, lane);
+  ring_load<TPW, 2>(r, wp, 2, act_lane, lane);
+  for (int j = 0; j < kg; j += 4) {
+    // The scheduling barriers keep the compiler from sinking a prefetch below
+    // the MFMA block it is meant to overlap with.  Groups past the end reload
+    // the last one (valid memory, unused values).
+    ring_load<TPW, 3>(r, wp, min(j + 3, last), act_lane, lane);
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-#pragma unroll
-      for (int t = 0; t < TPW; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[t][e], xa[e], acc[t], 0, 0, 0);
+    ring_mfma<TPW, 0>(r, acc);
     __builtin_amdgcn_sched_barrier(0);
-    {
-      const int jn = (j + 2 < kg) ? (j + 2) : j;  // last iteration reloads a valid group
-      const f32x4* p = wp + (size_t)jn * TPW * 64 + lane;
-#pragma unroll
-      for (int t = 0; t < TPW; ++t) wa[t] = p[t * 64];
-      xa = *reinterpret_cast<const f32x4*>(act_lane + 8 * jn);
-    }
+    ring_load<TPW, 0>(r, wp, min(j + 4, last), act_lane, lane);
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-#pragma unroll
-      for (int t = 0; t < TPW; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(wb[t][e], xb[e], acc[t], 0, 0, 0);
+    ring_mfma<TPW, 1>(r, acc);
+    __builtin_amdgcn_sched_barrier(0);
+    ring_load<TPW, 1>(r, wp, min(j + 5, last), act_lane, lane);
+    __builtin_amdgcn_sched_barrier(0);
+    ring_mfma<TPW, 2>(r, acc);
+    __builtin_amdgcn_sched_barrier(0);
+    ring_load<TPW, 2>(r, wp, min(j + 6, last), act_lane, lane);
+    __builtin_amdgcn_sched_barrier(0);
+    ring_mfma<TPW, 3>(r, acc);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
@@ -198,7 +215,7 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
   }
 }
 
-constexpr int kWaves = 8;
+constexpr int kWaves = 4;  // one wave per SIMD: measured faster than two (fewer, longer MFMA runs between load bursts)
 constexpr size_t kLdsBytes = (size_t)(kRows * kStride + (kWaves * 64 / 32) * 32) * sizeof(float);
 
 }  // namespace
@@ -259,7 +276,7 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
   }
   for (int i = 0; i < hidden_layers + 2; ++i)
     if (W[i] == nullptr || b[i] == nullptr) { *err = HBT_EINVAL; return nullptr; }
-  const int in_padded = (int)align_up((size_t)in_features, 16);
+  const int in_padded = (int)align_up((size_t)in_features, 32);
   if (width != kWidth || in_padded > kMaxInPadded || hidden_layers > 64) {
     *err = HBT_ESIZE;
     return nullptr;
