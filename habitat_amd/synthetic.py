@@ -141,3 +141,101 @@ def mlp_features(kind, n, seed=2, device_features=None):
     mu = np.mean(x, axis=0)
     sigma = np.std(x, axis=0)
     return np.ascontiguousarray(x), mu, sigma
+
+
+def resnet50_trace(origin, batch=32, seed=3, metrics_fraction=0.3):
+    """A ResNet-50-shaped training-iteration trace measured on `origin`: 53
+    conv2d and 1 linear operation (MLP-predicted), and the batch-norm, ReLU,
+    pooling, residual-add, loss and optimizer operations around them
+    (wave-scaled; forward and backward kernels).  Shapes follow the torchvision
+    layer table; times and metrics are synthetic but consistent with the shapes.
+    About 180 operations and 900 kernel records."""
+    from habitat_amd.analysis.arguments import Arguments
+    from habitat_amd.analysis.kernels import KernelInstance, MeasuredKernel
+    from habitat_amd.analysis.operation import MeasuredOperation
+    from habitat_amd.analysis.run_time import RunTimeMeasurement
+    from habitat_amd.analysis.trace import Trace
+
+    rng = np.random.default_rng(seed)
+    bw = origin.mem_bandwidth_gb * 1e9
+    peak = origin.peak_gflops_per_second * 1e9
+    ops = []
+
+    def kernel(name, elements, bytes_per_el=8.0, block=256, regs=None):
+        nblocks = max(1, int(np.ceil(elements / (block * 4))))
+        t_ns = max(1500, int(elements * bytes_per_el / (bw * rng.uniform(0.45, 0.8)) * 1e9))
+        k = KernelInstance(name, nblocks, block, 0, int(rng.choice([0, 0, 0, 2048, 4096])),
+                           int(regs if regs is not None else rng.integers(16, 48)), t_ns)
+        metrics = []
+        if rng.random() < metrics_fraction:
+            rd = elements * bytes_per_el * rng.uniform(0.4, 0.6)
+            m = KernelInstance(name, nblocks, block, 0, 0, k.metadata["registers_per_thread"], t_ns, [
+                ("dram__bytes_read.sum", float(int(rd))),
+                ("dram__bytes_write.sum", float(int(elements * bytes_per_el - rd))),
+                ("smsp__sass_thread_inst_executed_ops_fadd_fmul_ffma_pred_on.avg."
+                 "pct_of_peak_sustained_elapsed", float(rng.uniform(0.5, 12.0)))])
+            metrics = [m]
+        return MeasuredKernel(k, metrics, origin)
+
+    def scaled_op(name, elements, n_fwd, n_bwd):
+        def one_pass(tag, count):
+            ks = [kernel("%s_%s_%d" % (name, tag, i), elements) for i in range(count)]
+            total_ms = sum(k.run_time_ns for k in ks) / 1e6 + rng.uniform(0.004, 0.02) * count
+            return RunTimeMeasurement(total_ms, ks, origin)
+        fwd = one_pass("fwd", n_fwd)
+        bwd = one_pass("bwd", n_bwd) if n_bwd else None
+        ops.append(MeasuredOperation(name, Arguments((), {}), fwd, bwd, origin))
+
+    def conv(cin, cout, k, stride, hw_in, bias=False):
+        pad = k // 2
+        hw_out = (hw_in + 2 * pad - k) // stride + 1
+        flops = 2.0 * batch * cout * hw_out * hw_out * cin * k * k
+        fwd_ms = flops / (peak * rng.uniform(0.35, 0.7)) * 1e3 + 0.02
+        args = ((batch, cin, hw_in, hw_in), (cout, cin, k, k), (cout,) if bias else None,
+                (stride, stride), (pad, pad), (1, 1), 1)
+        ops.append(MeasuredOperation(
+            "conv2d", Arguments(args, {}), RunTimeMeasurement(fwd_ms, [], origin),
+            RunTimeMeasurement(2.1 * fwd_ms, [], origin), origin))
+        return hw_out
+
+    def bn_relu(c, hw, relu=True):
+        el = batch * c * hw * hw
+        scaled_op("batch_norm", el, 3, 5)
+        if relu:
+            scaled_op("relu_", el, 1, 1)
+
+    hw = conv(3, 64, 7, 2, 224)
+    bn_relu(64, hw)
+    scaled_op("max_pool2d", batch * 64 * hw * hw, 1, 1)
+    hw = (hw + 2 - 3) // 2 + 1
+    cin = 64
+    for stage, (blocks, width) in enumerate(zip([3, 4, 6, 3], [64, 128, 256, 512])):
+        for b in range(blocks):
+            stride = 2 if (b == 0 and stage > 0) else 1
+            conv(cin, width, 1, 1, hw)
+            bn_relu(width, hw)
+            hw2 = conv(width, width, 3, stride, hw)
+            bn_relu(width, hw2)
+            conv(width, width * 4, 1, 1, hw2)
+            bn_relu(width * 4, hw2, relu=False)
+            if b == 0:
+                conv(cin, width * 4, 1, stride, hw)
+                bn_relu(width * 4, hw2, relu=False)
+            el = batch * width * 4 * hw2 * hw2
+            scaled_op("add_", el, 1, 2)
+            scaled_op("relu_", el, 1, 1)
+            cin, hw = width * 4, hw2
+    scaled_op("adaptive_avg_pool2d", batch * cin * hw * hw, 1, 1)
+    fwd_ms = 2.0 * batch * 2048 * 1000 / (peak * 0.5) * 1e3 + 0.02
+    ops.append(MeasuredOperation(
+        "linear", Arguments(((batch, 2048), (1000, 2048), (1000,)), {}),
+        RunTimeMeasurement(fwd_ms, [], origin), RunTimeMeasurement(2 * fwd_ms, [], origin), origin))
+    scaled_op("log_softmax", batch * 1000, 1, 1)
+    scaled_op("nll_loss", batch * 1000, 1, 1)
+    # optimizer step: two small kernels per parameter tensor, no backward pass
+    step = [kernel("sgd_%d" % i, int(rng.integers(64, 2_400_000)), 12.0) for i in range(322)]
+    ops.append(MeasuredOperation(
+        "_foreach_add_", Arguments((), {}),
+        RunTimeMeasurement(sum(k.run_time_ns for k in step) / 1e6 * 1.1, step, origin), None,
+        origin))
+    return Trace(origin, ops)

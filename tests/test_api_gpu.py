@@ -1,0 +1,216 @@
+"""GPU: the host-side mirror of the reference's analysis API — scalar
+wave-scaling strategies with the reference's exceptions, the Predictor routing
+and the trace-level sums — against the CPU oracle."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import oracle_device
+from habitat_amd import Device, synthetic
+from habitat_amd.analysis.kernels import KernelInstance, MeasuredKernel, PredictedKernel
+from habitat_amd.analysis.metrics import Metric
+from habitat_amd.analysis.mlp.mlp import RuntimePredictor
+from habitat_amd.analysis.predictor import Predictor
+from habitat_amd.analysis.trace import Trace
+from habitat_amd.analysis.wave_scaling.metadata import NullMetadataManager
+from habitat_amd.analysis.wave_scaling.resimplified import resimplified_wave_scaling
+from habitat_amd.analysis.wave_scaling.roofline import roofline_wave_scaling
+from habitat_amd.analysis.wave_scaling.unified import unified_wave_scaling
+from oracle import mlp as omlp
+from oracle import predictor as opred
+from oracle import wave_scaling as ows
+
+pytestmark = pytest.mark.gpu
+
+
+def odev(d):
+    return oracle_device(d.as_dict())
+
+
+def make_kernel(device, num_blocks=4096, block=256, dyn=0, stat=0, regs=32, t_ns=1000000,
+                metrics=(50.0, 1e8, 1e8), name="k"):
+    k = KernelInstance(name, num_blocks, block, dyn, stat, regs, t_ns)
+    mk = []
+    if metrics is not None:
+        eff, rd, wr = metrics
+        mk = [KernelInstance(name, num_blocks, block, dyn, stat, regs, t_ns, [
+            ("flop_sp_efficiency", eff), ("dram_read_bytes", rd), ("dram_write_bytes", wr)])]
+    return MeasuredKernel(k, mk, device)
+
+
+def as_record(kernel, metrics):
+    md = kernel.metadata
+    eff, rd, wr = metrics if metrics is not None else (0.0, 0.0, 0.0)
+    return dict(num_blocks=kernel.num_blocks, block_size=md["block_size"],
+                dynamic_smem=md["dynamic_shared_memory"], static_smem=md["static_shared_memory"],
+                regs_per_thread=md["registers_per_thread"], run_time_ns=kernel.run_time_ns,
+                flop_sp_efficiency=eff, dram_read_bytes=rd, dram_write_bytes=wr)
+
+
+class TableManager:
+    """A metadata manager backed by a dict, to exercise dest_regs."""
+
+    def __init__(self, table):
+        self.table = table
+
+    def kernel_registers_for(self, kernel, device):
+        return self.table.get((kernel.name, device.name))
+
+
+def test_scalar_strategies_known_answers(kat):
+    mm = NullMetadataManager()
+    for row in kat["scaling"]:
+        o, d = getattr(Device, row["origin"]), getattr(Device, row["dest"])
+        k = make_kernel(o, num_blocks=row["num_blocks"])
+        for strategy in (unified_wave_scaling, roofline_wave_scaling):
+            p = strategy(k, o, d, mm)
+            assert isinstance(p, PredictedKernel) and p.name == "k"
+            assert p.run_time_ns == pytest.approx(row["time_ns"], rel=1e-6)
+    # no metrics: unified falls back, roofline raises AttributeError like the reference
+    k = make_kernel(Device.V100, metrics=None)
+    assert unified_wave_scaling(k, Device.V100, Device.P100, mm).run_time_ns == pytest.approx(
+        1e6 * 739 / 501, rel=1e-12)
+    assert resimplified_wave_scaling(k, Device.V100, Device.P100, mm).run_time_ns == pytest.approx(
+        1e6 * 739 / 501, rel=1e-12)
+    with pytest.raises(AttributeError, match="Unknown metric"):
+        roofline_wave_scaling(k, Device.V100, Device.P100, mm)
+    small = make_kernel(Device.V100, num_blocks=3, metrics=None)
+    assert resimplified_wave_scaling(small, Device.V100, Device.P100, mm).run_time_ns == 1000000
+
+
+def test_scalar_strategies_raise_what_the_reference_raises():
+    mm = NullMetadataManager()
+    v100, p100, mi = Device.V100, Device.P100, Device.MI355X
+    with pytest.raises(ZeroDivisionError):      # origin cannot hold the block
+        unified_wave_scaling(make_kernel(v100, 100, 1024, regs=255), v100, p100, mm)
+    with pytest.raises(ZeroDivisionError):      # destination cannot, kernel small on origin
+        unified_wave_scaling(make_kernel(mi, 10, dyn=60000), mi, v100, mm)
+    big = unified_wave_scaling(make_kernel(mi, 1 << 16, dyn=60000), mi, v100, mm)
+    assert big.run_time_ns > 0                  # short-circuit: no exception
+    with pytest.raises(AssertionError):         # gamma > 1
+        roofline_wave_scaling(make_kernel(v100, 100, metrics=(50.0, -3e8, 1e8)), v100, p100, mm)
+    with pytest.raises(ZeroDivisionError):      # num_blocks == 0
+        roofline_wave_scaling(make_kernel(v100, 0), v100, p100, mm)
+    assert resimplified_wave_scaling(make_kernel(v100, 0, metrics=None), v100, p100,
+                                     mm).run_time_ns == 1000000
+
+
+def test_scalar_strategy_uses_the_register_table():
+    k = make_kernel(Device.V100, num_blocks=400, name="gemm")
+    rec = as_record(k, (50.0, 1e8, 1e8))
+    mm = TableManager({("gemm", "P100"): 128})
+    got = unified_wave_scaling(k, Device.V100, Device.P100, mm).run_time_ns
+    want = ows.unified(rec, odev(Device.V100), odev(Device.P100), dest_regs=128)
+    assert got == pytest.approx(want, rel=1e-6)
+    # with 128 registers the P100 wave is 112 blocks instead of 448: 400 blocks are no longer "small"
+    other = unified_wave_scaling(k, Device.V100, Device.P100, NullMetadataManager()).run_time_ns
+    assert other != pytest.approx(want, rel=1e-3)
+
+
+def seeded_predictors():
+    preds = {}
+    for kind in ("conv2d", "linear", "bmm", "lstm"):
+        torch.manual_seed(0)
+        rp = RuntimePredictor(kind, 8, 1024)
+        x, mu, sigma = synthetic.mlp_features(kind, 2048, seed=2)
+        rp.set_normalization(mu, sigma)
+        preds[kind] = rp
+    return preds
+
+
+def oracle_operation_ms(op, dest, preds):
+    """Predicted time of one operation by the oracle modules."""
+    from habitat_amd.analysis import predictor as P
+    o, d = odev(op.device), odev(dest)
+    if op.name in ("conv2d", "linear", "bmm", "lstm"):
+        rp = preds[op.name]
+        a = P._ARGUMENTS[op.name](op)
+        feats = [a[x] for x in rp.model.features]
+        from habitat_amd.analysis.mlp.devices import get_device_features
+        rows = np.array([feats + get_device_features(dest.name, rp.device_params),
+                         feats + get_device_features(op.device.name, rp.device_params)], np.float64)
+        y = omlp.forward_fp64(rp.model.state_dict(), rows, rp.mu, rp.sigma)
+        return opred.special_op_ms(op.run_time_ms, y[0], y[1])
+    total = 0.0
+    for rt in (op.forward, op.backward):
+        if rt is None:
+            continue
+        pred = []
+        for k in rt.kernels:
+            try:
+                m = tuple(k.get_metric(x) for x in (Metric.SinglePrecisionFLOPEfficiency,
+                                                    Metric.DRAMReadBytes, Metric.DRAMWriteBytes))
+            except AttributeError:
+                m = None
+            pred.append(ows.unified(as_record(k, m), o, d, has_metrics=m is not None))
+        total += opred.wave_scaled_pass_ms(rt.run_time_ms, [k.run_time_ns for k in rt.kernels], pred)
+    return total
+
+
+def test_predictor_on_resnet50_shaped_trace():
+    origin, dest = Device.V100, Device.T4
+    trace = synthetic.resnet50_trace(origin, batch=16, seed=3)
+    preds = seeded_predictors()
+    predictor = Predictor(mlp_predictors=preds)
+    predicted = trace.to_device(dest, predictor)
+    assert isinstance(predicted, Trace) and predicted.device is dest
+    assert len(predicted.operations) == len(trace.operations)
+    want = [oracle_operation_ms(op, dest, preds) for op in trace.operations]
+    got = [op.run_time_ms for op in predicted.operations]
+    for op, g, w in zip(trace.operations, got, want):
+        tol = 1e-4 if op.name in ("conv2d", "linear") else 1e-6
+        assert g == pytest.approx(w, rel=tol), op.name
+    assert predicted.run_time_ms == pytest.approx(opred.trace_ms(want), rel=1e-5)
+    # one operation at a time gives the same numbers as the batched call
+    for idx in (0, 1, 5, len(trace.operations) - 1):
+        single = predictor.predict_operation(trace.operations[idx], dest)
+        assert single.run_time_ms == pytest.approx(got[idx], rel=1e-12)
+    assert trace.to_device(origin, predictor) is trace
+    with pytest.raises(RuntimeError):
+        predicted.operations[0].to_device(origin, predictor)
+
+
+def test_predictor_with_a_caller_supplied_strategy_and_pass_through_ops():
+    from habitat_amd.analysis.arguments import Arguments
+    from habitat_amd.analysis.operation import MeasuredOperation
+    from habitat_amd.analysis.run_time import RunTimeMeasurement
+    origin, dest = Device.V100, Device.P100
+    calls = []
+
+    def halve(kernel, origin_device, dest_device, metadata_manager):
+        calls.append(kernel.name)
+        return PredictedKernel(kernel, kernel.run_time_ns / 2)
+
+    ks = [make_kernel(origin, name="a", t_ns=2000000), make_kernel(origin, name="b", t_ns=1000000)]
+    op = MeasuredOperation("relu_", Arguments((), {}), RunTimeMeasurement(3.5, ks, origin), None, origin)
+    gru = MeasuredOperation("gru", Arguments((), {}), RunTimeMeasurement(7.0, [], origin),
+                            RunTimeMeasurement(9.0, [], origin), origin)
+    p = Predictor(wave_scaling_strategy=halve)
+    out = p.predict_operations([op, gru], dest)
+    assert calls == ["a", "b"]
+    assert out[0].run_time_ms == pytest.approx((0.5e6 + 1.5e6) / 1e6)   # overhead kept, kernels halved
+    assert out[1].run_time_ms == 16.0                                     # no predictor: unscaled
+    # kernels longer than the measured pass: overhead clamps at zero
+    op2 = MeasuredOperation("relu_", Arguments((), {}), RunTimeMeasurement(1.0, ks, origin), None, origin)
+    assert p.predict_operation(op2, dest).run_time_ms == pytest.approx(1.5)
+
+
+def test_device_sweep_matches_per_device_prediction():
+    origin = Device.V100
+    trace = synthetic.resnet50_trace(origin, batch=8, seed=5)
+    preds = seeded_predictors()
+    predictor = Predictor(mlp_predictors=preds)
+    devices, feats = synthetic.device_sweep(24, seed=1)
+    from habitat_amd.analysis.mlp import devices as md
+    for d, f in zip(devices, feats):
+        md.register_device(d.name, *f)
+    totals = trace.to_devices(devices, predictor)
+    assert len(totals) == 24
+    for i in (0, 7, 23):
+        want = trace.to_device(devices[i], predictor).run_time_ms
+        assert totals[i] == pytest.approx(want, rel=1e-9)
+    oracle_total = opred.trace_ms([oracle_operation_ms(op, devices[3], preds)
+                                   for op in trace.operations])
+    assert totals[3] == pytest.approx(oracle_total, rel=1e-5)

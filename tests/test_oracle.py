@@ -228,3 +228,22 @@ def test_python_restatement_over_compiled_reference_occupancy(kat):
         o, d = oracle_device(DEVS[row["origin"]]), oracle_device(DEVS[row["dest"]])
         rec = _record(kat, row["num_blocks"])
         assert ows.unified(rec, o, d, occupancy=ref_occ) == pytest.approx(row["time_ns"], rel=1e-14)
+
+
+def test_predictor_arithmetic():
+    """oracle/predictor.py against a three-operation, five-kernel trace worked
+    by hand."""
+    from oracle import predictor as opred
+    # op 1: forward 2.0 ms with kernels 0.5 + 0.75 ms -> overhead 0.75 ms; the
+    # kernels are predicted at 0.25 + 0.5 ms -> 1.5 ms.  Backward 1.0 ms with one
+    # 1.5 ms kernel (longer than the pass: overhead clamps to 0) predicted 3.0 ms.
+    fwd = opred.wave_scaled_pass_ms(2.0, [500000, 750000], [250000.0, 500000.0])
+    bwd = opred.wave_scaled_pass_ms(1.0, [1500000], [3000000.0])
+    assert fwd == 1.5 and bwd == 3.0
+    # op 2: 4 ms measured, MLP predicts 0.02 on the destination, 0.05 on the origin
+    assert opred.special_op_ms(4.0, 0.02, 0.05) == pytest.approx(1.6)
+    # op 3: a negative prediction is clamped to zero
+    assert opred.special_op_ms(4.0, -0.02, 0.05) == 0.0
+    assert opred.trace_ms([fwd + bwd, 1.6, 0.0]) == pytest.approx(6.1)
+    # a pass without kernels keeps its measured time
+    assert opred.wave_scaled_pass_ms(0.7, [], []) == pytest.approx(0.7)
