@@ -304,9 +304,15 @@ class Predictor:
         return self._scale_with("lstm", operation, dest_device)
 
     # ------------------------------------------------------- device sweeps
-    def predict_trace_times(self, trace, dest_devices):
+    def predict_trace_times(self, trace, dest_devices, device_features=None):
         """Predicted iteration time [ms] of `trace` on every device of
         `dest_devices` (the sum of analysis/trace.py:27-36 over predicted
         operations).  Kernel records are scaled for all destinations at once."""
         from habitat_amd.analysis.sweep import predict_trace_times
-        return predict_trace_times(self, trace, dest_devices)
+        return predict_trace_times(self, trace, dest_devices, device_features)
+
+    def predict_trace_sweep(self, trace, dest_devices, device_features=None):
+        """Like predict_trace_times, with the per-pass and per-operation pieces
+        (a habitat_amd.analysis.sweep.TraceSweep)."""
+        from habitat_amd.analysis.sweep import predict_trace_sweep
+        return predict_trace_sweep(self, trace, dest_devices, device_features)

@@ -43,8 +43,10 @@ class Trace:
         predictor = predictor if predictor is not None else Trace.default_predictor()
         return Trace(dest_device, predictor.predict_operations(self._operations, dest_device))
 
-    def to_devices(self, dest_devices, predictor=None):
+    def to_devices(self, dest_devices, predictor=None, device_features=None):
         """Predicted run time [ms] of the whole trace on each device of a sweep,
-        computed on the GPU; returns a list of floats."""
+        computed on the GPU; returns a list of floats.  `device_features` maps
+        device names to their four MLP features where the built-in table has
+        none."""
         predictor = predictor if predictor is not None else Trace.default_predictor()
-        return predictor.predict_trace_times(self, dest_devices)
+        return predictor.predict_trace_times(self, dest_devices, device_features)

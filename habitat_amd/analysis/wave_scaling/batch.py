@@ -124,3 +124,84 @@ def wave_scale(records, origin, dests, out=None, stream=None, waves=True, status
             _ptr(out.wave_dest), _ptr(out.status), ctypes.c_void_p(stream.cuda_stream))
     _lib.check(rc, "hbt_wave_scale")
     return out
+
+
+class DeviceTable:
+    """A sweep of destination devices resident on the GPU (`hbt_device_table`)."""
+
+    def __init__(self, origin, dests):
+        self.origin = origin
+        self.dests = list(dests)
+        if not self.dests:
+            raise ValueError("a device table needs at least one destination")
+        specs = (_lib.DeviceSpec * len(self.dests))(*[d.spec for d in self.dests])
+        err = ctypes.c_int(0)
+        self.torch_device = torch.device("cuda", torch.cuda.current_device())
+        self.handle = _lib.lib().hbt_device_table_create(
+            ctypes.byref(origin.spec), specs, len(self.dests), ctypes.byref(err))
+        if not self.handle:
+            raise _lib.HabitatLibraryError(err.value, "hbt_device_table_create")
+
+    def __len__(self):
+        return len(self.dests)
+
+    def __del__(self):
+        try:
+            if getattr(self, "handle", None):
+                _lib.lib().hbt_device_table_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+def wave_scale_sum(records, table, segment=None, n_segments=1, stream=None):
+    """Per destination of `table` and per segment, the sum of the scaled times
+    of `records` (see hbt_wave_scale_sum).  `segment`: int32 GPU tensor [n] or
+    None.  Returns (sums [n_dest, n_segments] float64, bad [n_dest] int32), both
+    GPU tensors, not synchronised."""
+    if records.device != table.torch_device:
+        raise ValueError("records and device table live on different GPUs")
+    if segment is not None and (segment.dtype != torch.int32 or segment.shape != (records.n,)
+                                or segment.device != records.device):
+        raise TypeError("segment must be an int32 GPU tensor of length %d" % records.n)
+    n_dest = len(table)
+    sums = torch.empty((n_dest, n_segments), dtype=torch.float64, device=records.device)
+    bad = torch.empty((n_dest,), dtype=torch.int32, device=records.device)
+    if stream is None:
+        stream = torch.cuda.current_stream(records.device)
+    c = records.columns
+    with torch.cuda.device(records.device):
+        rc = _lib.lib().hbt_wave_scale_sum(
+            table.handle, records.n,
+            _ptr(c["num_blocks"]), _ptr(c["block_size"]), _ptr(c["dynamic_smem"]),
+            _ptr(c["static_smem"]), _ptr(c["regs_per_thread"]), _ptr(records.dest_regs),
+            _ptr(c["run_time_ns"]), _ptr(c["flop_sp_efficiency"]), _ptr(c["dram_read_bytes"]),
+            _ptr(c["dram_write_bytes"]), _ptr(records.has_metrics),
+            _ptr(segment.contiguous() if segment is not None else None), n_segments,
+            _ptr(sums), _ptr(bad), ctypes.c_void_p(stream.cuda_stream))
+    _lib.check(rc, "hbt_wave_scale_sum")
+    return sums, bad
+
+
+def ratio_scale(pred, run_time_ms, n_dest, totals=None, want_ms=True, stream=None):
+    """MLP-predicted operations on a sweep (see hbt_ratio_scale).  pred: float32
+    GPU tensor [(n_dest + 1), n_ops] whose last row is the origin; run_time_ms:
+    float64 GPU tensor [n_ops].  Returns ms [n_dest, n_ops] (or None) and adds the
+    per-destination sums to `totals` ([n_dest] float64) if given."""
+    n_ops = run_time_ms.shape[0]
+    if pred.dtype != torch.float32 or tuple(pred.shape) != (n_dest + 1, n_ops):
+        raise TypeError("pred must be float32 [%d, %d]" % (n_dest + 1, n_ops))
+    if run_time_ms.dtype != torch.float64 or (totals is not None and (
+            totals.dtype != torch.float64 or totals.shape != (n_dest,))):
+        raise TypeError("run_time_ms and totals must be float64")
+    pred = pred.contiguous()
+    out = (torch.empty((n_dest, n_ops), dtype=torch.float64, device=pred.device)
+           if want_ms else None)
+    if stream is None:
+        stream = torch.cuda.current_stream(pred.device)
+    with torch.cuda.device(pred.device):
+        rc = _lib.lib().hbt_ratio_scale(_ptr(pred), n_dest, n_ops, _ptr(run_time_ms.contiguous()),
+                                        _ptr(out), _ptr(totals),
+                                        ctypes.c_void_p(stream.cuda_stream))
+    _lib.check(rc, "hbt_ratio_scale")
+    return out

@@ -12,6 +12,14 @@
 
 namespace hbt {
 
+OriginArgs make_origin_args(const hbt_device_spec& o) {
+  OriginArgs a{};
+  a.dev = make_occ_device(o);
+  a.peak_gflops = o.peak_gflops;
+  a.inv_sms = 1.0f / (float)o.num_sms;
+  return a;
+}
+
 DestArgs make_dest_args(const hbt_device_spec& o, const hbt_device_spec& d) {
   DestArgs p{};
   p.dev = make_occ_device(d);
@@ -163,9 +171,7 @@ int hbt_wave_scale(const hbt_device_spec* origin, const hbt_device_spec* dests, 
   a.dram_read_bytes = dram_read_bytes; a.dram_write_bytes = dram_write_bytes;
   a.has_metrics = has_metrics;
   a.out_occ_origin = out_occ_origin; a.out_wave_origin = out_wave_origin;
-  a.origin = make_occ_device(*origin);
-  a.origin_peak_gflops = origin->peak_gflops;
-  a.origin_inv_sms = 1.0f / (float)origin->num_sms;
+  a.origin = make_origin_args(*origin);
 
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
   for (int32_t d0 = 0; d0 < n_dest; d0 += kMaxDestPerLaunch) {

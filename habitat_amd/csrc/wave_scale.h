@@ -27,6 +27,13 @@ struct DestArgs {
   float inv_sms;               // 1 / num_sms rounded to float
 };
 
+// The origin device's share of the constants.
+struct OriginArgs {
+  OccDevice dev;
+  double peak_gflops;  // origin.peak_gflops_per_second
+  float inv_sms;       // 1 / origin.num_sms rounded to float
+};
+
 struct WaveScaleArgs {
   int64_t n;
   int32_t n_dest;
@@ -48,12 +55,11 @@ struct WaveScaleArgs {
   int32_t* out_wave_origin;    // [n], nullable
   int32_t* out_wave_dest;      // [n_dest][n], nullable
   uint8_t* out_status;         // [n_dest][n], nullable
-  OccDevice origin;
-  double origin_peak_gflops;
-  float origin_inv_sms;        // 1 / origin.num_sms rounded to float
+  OriginArgs origin;
   DestArgs dest[kMaxDestPerLaunch];
 };
 
+OriginArgs make_origin_args(const hbt_device_spec& origin);
 DestArgs make_dest_args(const hbt_device_spec& origin, const hbt_device_spec& dest);
 
 // `vectorised` needs every column 16-byte aligned (and n % 4 == 0 when n_dest > 1).

@@ -24,191 +24,16 @@
 // Keep a*b+c as two roundings where the reference (CPython floats) has two.
 #pragma clang fp contract(off)
 
+#include "wave_scale_device.h"
+
 namespace hbt {
 
 namespace {
 
+using namespace dev;
+
 constexpr int kRecPerThread = 2;
 constexpr int kBlock = 256;
-
-// log2(i) for i = 0..32 (entry 0 unused), padded to one entry per lane.  A
-// kernel that fits in one wave on a device has num_blocks < num_sms * occupancy
-// with occupancy <= 32 block slots, so ceil(num_blocks / num_sms) is an integer
-// in 1..32 and the logarithm of the small-kernel factor needs no more than this
-// table.  Each wavefront keeps it in one register pair (lane i holds entry i)
-// and looks entries up with a cross-lane permute: no LDS, no barrier.
-__device__ const double kLog2Int[64] = {
-    0x0.0p+0, 0x0.0p+0, 0x1.0000000000000p+0, 0x1.95c01a39fbd68p+0, 0x1.0000000000000p+1,
-    0x1.2934f0979a371p+1, 0x1.4ae00d1cfdeb4p+1, 0x1.675767f54042dp+1, 0x1.8000000000000p+1,
-    0x1.95c01a39fbd68p+1, 0x1.a934f0979a371p+1, 0x1.bacea7c065d42p+1, 0x1.cae00d1cfdeb4p+1,
-    0x1.d9a802391e233p+1, 0x1.e75767f54042dp+1, 0x1.f414fdb498226p+1, 0x1.0000000000000p+2,
-    0x1.0598fdbeb244cp+2, 0x1.0ae00d1cfdeb4p+2, 0x1.0fde0b5c81340p+2, 0x1.149a784bcd1b9p+2,
-    0x1.191bba891f171p+2, 0x1.1d6753e032ea1p+2, 0x1.21820a01ac755p+2, 0x1.2570068e7ef5ap+2,
-    0x1.2934f0979a371p+2, 0x1.2cd4011c8f119p+2, 0x1.305013ab7ce0ep+2, 0x1.33abb3faa0216p+2,
-    0x1.36e9291eaa65bp+2, 0x1.3a0a7eda4c113p+2, 0x1.3d118d66c4d4ep+2, 0x1.4000000000000p+2};
-
-struct RecordIn {
-  int32_t nb, block, smem_total, regs, dest_regs;
-  bool metrics;
-  double t, eff, rd, wr;
-};
-
-// Destination-independent part of one record.
-struct RecordMid {
-  SmemAlloc smem;
-  int32_t occ_o, wave_o;
-  int32_t origin_max_occ;  // ceil(num_blocks / origin.num_sms) when small_o, else 0
-  bool small_o;            // num_blocks // origin_wave == 0
-  double num_gflops, total_gb;
-};
-
-// 2^x for finite x, relative error below 1e-13: split x = n + f with
-// |f| <= 1/2, evaluate e^(f ln 2) by its Taylor polynomial of degree 11
-// ((ln2 / 2)^12 / 12! < 7e-15) and scale by 2^n.
-__device__ __forceinline__ double exp2_poly(double x) {
-  const double n = rint(x);
-  const double z = (x - n) * 0x1.62e42fefa39efp-1;  // f * ln 2
-  double p = 1.0 / 39916800.0;
-  p = fma(p, z, 1.0 / 3628800.0);
-  p = fma(p, z, 1.0 / 362880.0);
-  p = fma(p, z, 1.0 / 40320.0);
-  p = fma(p, z, 1.0 / 5040.0);
-  p = fma(p, z, 1.0 / 720.0);
-  p = fma(p, z, 1.0 / 120.0);
-  p = fma(p, z, 1.0 / 24.0);
-  p = fma(p, z, 1.0 / 6.0);
-  p = fma(p, z, 0.5);
-  p = fma(p, z, 1.0);
-  p = fma(p, z, 1.0);
-  // |x| beyond the exponent range saturates through ldexp (inf or 0)
-  const double nc = fmin(fmax(n, -4096.0), 4096.0);
-  return ldexp(p, (int)nc);
-}
-
-// x / c for a compile-time constant c, correctly rounded like the IEEE
-// division it replaces: q = x * (1/c) is within an ulp of the quotient, the
-// remainder x - q*c is exact in an FMA, and adding remainder * (1/c) back
-// rounds to the nearest double (Markstein's correction; checked against `/`
-// on 4e8 operands for each constant used here).  Operands whose remainder
-// could underflow or overflow take the hardware sequence instead.
-template <class C>
-__device__ __forceinline__ double div_const(double x) {
-  constexpr double c = C::value, rc = 1.0 / C::value;
-  const double ax = fabs(x);
-  if (__builtin_expect((ax > 0x1p+900) || (ax < 0x1p-900 && ax != 0.0), 0)) return x / c;
-  const double q = x * rc;
-  const double r = fma(-q, c, x);
-  return fma(r, rc, q);
-}
-struct C100 { static constexpr double value = 100.0; };
-struct C1e9 { static constexpr double value = 1e9; };
-
-// FAST: every device of the launch has OccDevice::fast_ok, so the 32-bit model
-// applies to every record.  Otherwise the 64-bit model with real divisions runs
-// (devices with limits of 2^22 and more: not real hardware, but in the domain).
-template <bool FAST>
-__device__ __forceinline__ int32_t occupancy_dev(const OccDevice& d, int32_t block,
-                                                 int32_t smem_total, const SmemAlloc& sm,
-                                                 int32_t regs) {
-  regs &= 0xFFFF;  // uint16_t narrowing, cpp/src/cuda/kernel.h:108
-  if (FAST) return occupancy_fast(d, block, sm, regs);
-  return occupancy_core(d, block, smem_total, regs);
-}
-
-// ceil(nb / sms) for 0 <= nb < 32 * sms.  The reference takes math.ceil of the
-// fp64 quotient (roofline.py:33-38); for operands below 2^53 that quotient is an
-// integer only when the division is exact, so the integer ceiling is the same.
-// On a fast_ok device sms <= 2^14 and nb < 2^19: float(nb) * (1/sms) is within
-// 2^-18 of the quotient, which is either an integer or at least 2^-14 away from
-// one, so ceil(product - 2^-16) is the exact ceiling.
-template <bool FAST>
-__device__ __forceinline__ int32_t ceil_div_small(int32_t nb, int32_t sms, float inv_sms) {
-  if (FAST) return (int32_t)ceilf(fmaf(__int2float_rn(nb), inv_sms, -0x1p-16f));
-  return (int32_t)(((int64_t)nb + sms - 1) / sms);
-}
-
-template <bool FAST>
-__device__ __forceinline__ RecordMid origin_part(const WaveScaleArgs& a, const RecordIn& r) {
-  RecordMid m;
-  m.smem = smem_alloc(r.smem_total);
-  m.occ_o = occupancy_dev<FAST>(a.origin, r.block, r.smem_total, m.smem, r.regs);
-  m.wave_o = mul_small(a.origin.num_sms, m.occ_o);
-  m.small_o = r.nb >= 0 && r.nb < m.wave_o;
-  m.origin_max_occ =
-      ceil_div_small<FAST>(m.small_o ? r.nb : 0, a.origin.num_sms, a.origin_inv_sms);
-  // roofline.py:72-76, same operation order (the three divisions by 1024 are
-  // exact scalings)
-  m.total_gb = (r.rd + r.wr) / 1024 / 1024 / 1024;
-  const double gflops_per_second = div_const<C100>(r.eff) * a.origin_peak_gflops;
-  m.num_gflops = div_const<C1e9>(gflops_per_second * r.t);
-  return m;
-}
-
-struct RecordOut {
-  double t;
-  int32_t occ_d, wave_d;
-  uint8_t status;
-};
-
-// Written with selects rather than branches: the 64 records of a wavefront
-// take all paths between them anyway.
-// log2 of a small-kernel block count (0..32).  PERMUTE: read it from the lane
-// that holds it (needs all 64 lanes of the wavefront active); otherwise gather
-// it from the table in memory.
-template <bool PERMUTE>
-__device__ __forceinline__ double log2_count(double log2_lane, int32_t count) {
-  if (PERMUTE) return __shfl(log2_lane, count & 63);
-  return kLog2Int[count & 63];
-}
-
-template <bool FAST, bool PERMUTE>
-__device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn& r,
-                                               const RecordMid& m, double log2_lane) {
-  RecordOut o;
-  const int32_t regs_d = r.dest_regs >= 0 ? r.dest_regs : r.regs;
-  o.occ_d = occupancy_dev<FAST>(p.dev, r.block, r.smem_total, m.smem, regs_d);
-  o.wave_d = mul_small(p.dev.num_sms, o.occ_d);
-
-  // roofline.py:86-101.  With I = gflops / gb the reference takes
-  // 0.5 * R / I above the ridge point R and 1 - 0.5 / R * I below; both are
-  // formed here from one division by choosing its operands first.  The choice
-  // compares gflops with R * gb instead of I with R, which can differ only
-  // within an ulp of the ridge, where the two expressions agree (gamma = 1/2).
-  const bool above = m.total_gb > 0 && m.num_gflops > p.ridge * m.total_gb;
-  const double q = (above ? p.half_ridge * m.total_gb : m.num_gflops) /
-                   (above ? m.num_gflops : m.total_gb);
-  double gamma = above ? q : p.neg_half_over_ridge * q + 1.;
-  gamma = (m.total_gb == 0) ? 0. : gamma;
-  gamma = (m.num_gflops < 1e-9) ? 1. : gamma;
-  const bool bad_gamma = r.metrics && !(gamma >= 0 && gamma <= 1);
-
-  // `a // wave_o == 0 and a // wave_d == 0`: the second test, and its division
-  // by zero, happen only when the first holds (roofline.py:29-30).
-  const bool small = m.small_o && r.nb < o.wave_d;
-  const int32_t dest_max_occ = ceil_div_small<FAST>(small ? r.nb : 0, p.dev.num_sms, p.inv_sms);
-
-  int32_t status = HBT_ST_OK;
-  status = (r.metrics && small && m.origin_max_occ == 0) ? HBT_ST_ZERO_BLOCKS : status;
-  status = (m.small_o && o.wave_d == 0) ? HBT_ST_DEST_WAVE_ZERO : status;
-  status = (m.wave_o == 0) ? HBT_ST_ORIGIN_WAVE_ZERO : status;
-  status = bad_gamma ? HBT_ST_BAD_GAMMA : status;
-  o.status = (uint8_t)status;
-
-  // roofline.py:32-45: (clk_ratio * dest_max_occ / origin_max_occ)^(1-gamma), both
-  // counts in 1..32; roofline.py:48-64: bw^gamma * clk^(1-gamma) * sm^(1-gamma)
-  const double gamma_compl = 1.0 - gamma;
-  const double log2_small =
-      p.log2_clk + log2_count<PERMUTE>(log2_lane, dest_max_occ) -
-      log2_count<PERMUTE>(log2_lane, m.origin_max_occ);
-  const double exponent =
-      small ? gamma_compl * log2_small : gamma * p.log2_bw + gamma_compl * p.log2_clk_sm;
-  const double t_roofline = r.t * exp2_poly(exponent);
-  // resimplified.py:25-40
-  const double t_plain = small ? r.t : r.t * p.bw_ratio;
-  const double t = r.metrics ? t_roofline : t_plain;
-  o.t = (status == HBT_ST_OK) ? t : __builtin_nan("");
-  return o;
-}
 
 template <class T, int N>
 struct alignas(sizeof(T) * N) Pack { T v[N]; };
@@ -265,7 +90,7 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, int64_t i) {
   for (int k = 0; k < R; ++k) {
     rin[k] = RecordIn{nb[k], block[k], smem_sum(stat[k], dyn[k]), regs[k], dregs[k],
                       hm[k] != 0, t[k], eff[k], rd[k], wr[k]};
-    mid[k] = origin_part<FAST>(a, rin[k]);
+    mid[k] = origin_part<FAST>(a.origin, rin[k]);
   }
 
   if (a.write_origin) {
@@ -322,7 +147,7 @@ void launch(const WaveScaleArgs& args, hipStream_t stream) {
 
 hipError_t launch_wave_scale(const WaveScaleArgs& args, bool vectorised, hipStream_t stream) {
   if (args.n <= 0) return hipSuccess;
-  bool fast = args.origin.fast_ok();
+  bool fast = args.origin.dev.fast_ok();
   for (int d = 0; d < args.n_dest; ++d) fast = fast && args.dest[d].dev.fast_ok();
   if (vectorised) {
     if (fast) launch<kRecPerThread, true>(args, stream);

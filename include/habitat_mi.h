@@ -8,6 +8,7 @@
  * and the call returns without synchronising.  Functions return 0 or a
  * negative HBT_E* code; hbt_strerror() names it.  There is no global state and
  * no CPU fallback: without a GPU the compute entry points return HBT_EHIP.
+ * Only the two *_create calls allocate device memory.
  *
  * Each entry point cites the reference interface it stands in for
  * (paths relative to the reference tree).
@@ -29,7 +30,7 @@ enum {
   HBT_EINVAL = -1, /* null pointer, negative count, bad argument */
   HBT_ESPEC = -2,  /* device spec outside the supported domain (see hbt_device_spec_check) */
   HBT_EHIP = -3,   /* a HIP runtime call failed (no GPU, bad stream, launch error) */
-  HBT_ENOMEM = -4, /* device allocation failed (hbt_mlp_create only) */
+  HBT_ENOMEM = -4, /* allocation failed (the *_create calls only) */
   HBT_EALIGN = -5, /* a column pointer is not aligned to its element size */
   HBT_ESIZE = -6   /* size beyond what the entry point supports */
 };
@@ -136,15 +137,65 @@ int hbt_wave_scale(const hbt_device_spec *origin, const hbt_device_spec *dests, 
                    void *hip_stream);
 
 /*
+ * A set of destination devices resident on the GPU, for predicting one trace
+ * on many devices at once.  hbt_device_table_create takes HOST pointers, folds
+ * the per-device constants of (origin, dests[i]) and uploads them to the
+ * current HIP device; with hbt_mlp_create it is the only call that allocates.
+ * Returns NULL on failure (and sets *err if err is not NULL).  No counterpart
+ * in the reference, which handles one destination per Trace.to_device call
+ * (analyzer/habitat/analysis/trace.py:38-51).
+ */
+typedef struct hbt_device_table hbt_device_table;
+hbt_device_table *hbt_device_table_create(const hbt_device_spec *origin,
+                                          const hbt_device_spec *dests, int32_t n_dest, int *err);
+int32_t hbt_device_table_size(const hbt_device_table *table);
+void hbt_device_table_destroy(hbt_device_table *table);
+
+/*
+ * Wave scaling fused with the per-pass sums: for every destination d of the
+ * table and every segment s, out_sum[d][s] = sum of the scaled times of the
+ * records k with segment[k] == s.  A segment is one forward or backward pass of
+ * one operation, so out_sum is the kernel part of RunTimePrediction.run_time_ms
+ * (analyzer/habitat/analysis/run_time.py:50-58) for the kernels that
+ * Predictor._wave_scale (analysis/predictor.py:111-130) scales one by one; the
+ * caller adds the pass overhead, which does not depend on the destination.
+ * Input columns as for hbt_wave_scale; `segment` (device, [n], nullable = one
+ * segment) holds values in [0, n_segments), others are ignored.  Records whose
+ * status is not HBT_ST_OK on d add nothing and are counted in out_bad[d]
+ * (nullable): the reference would have raised for that destination.  out_sum
+ * ([n_dest][n_segments]) and out_bad ([n_dest]) are overwritten.  Sums are
+ * accumulated with floating-point atomics: their rounding can differ in the
+ * last bits from run to run.  Must be called with the table's device current.
+ */
+int hbt_wave_scale_sum(const hbt_device_table *table, int64_t n, const int32_t *num_blocks,
+                       const int32_t *block_size, const int32_t *dynamic_smem,
+                       const int32_t *static_smem, const int32_t *regs, const int32_t *dest_regs,
+                       const double *run_time_ns, const double *flop_sp_efficiency,
+                       const double *dram_read_bytes, const double *dram_write_bytes,
+                       const uint8_t *has_metrics, const int32_t *segment, int32_t n_segments,
+                       double *out_sum, int32_t *out_bad, void *hip_stream);
+
+/*
+ * The last step of the MLP-predicted operations for a device sweep
+ * (analysis/predictor.py:132-148 with :182,218,238,283): pred is
+ * [(n_dest + 1)][n_ops] fp32 MLP outputs, the last row evaluated with the
+ * origin's device features; out_ms[d][o] = run_time_ms[o] * pred[d][o] /
+ * pred[n_dest][o] in fp64, negative values replaced by 0 (out_ms nullable), and
+ * out_total[d] += sum over o of out_ms[d][o] (nullable).
+ */
+int hbt_ratio_scale(const float *pred, int32_t n_dest, int32_t n_ops, const double *run_time_ms,
+                    double *out_ms, double *out_total, void *hip_stream);
+
+/*
  * Per-operation MLP (fc1 -> ReLU -> hidden x (Linear, ReLU) -> fc2), the
  * network of analysis/mlp/mlp.py:17-109.  hbt_mlp_create takes HOST pointers:
  * W[0] is fc1.weight [width][in_features], W[1..hidden] are the hidden
  * weights [width][width], W[hidden+1] is fc2.weight [1][width], all row-major
  * fp32 as in a torch state_dict; b[] likewise; mu and sigma are the
  * checkpoint's normalisation vectors [in_features] (mlp.py:133-137).  The
- * weights are copied to the current HIP device in the layout the kernels want;
- * this is the only call that allocates.  Returns NULL on failure (and sets
- * *err if err is not NULL).
+ * weights are copied to the current HIP device in the layout the kernels want
+ * (this call and hbt_device_table_create are the only ones that allocate).
+ * Returns NULL on failure (and sets *err if err is not NULL).
  */
 typedef struct hbt_mlp hbt_mlp;
 hbt_mlp *hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layers,

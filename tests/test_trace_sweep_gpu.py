@@ -1,0 +1,163 @@
+"""GPU: the fused per-pass sums (hbt_wave_scale_sum), the ratio kernel
+(hbt_ratio_scale) and the 256-device sweep of BASELINE's end-to-end
+configuration, against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import oracle_device
+from habitat_amd import Device, DeviceProperties, _lib, synthetic
+from habitat_amd.analysis.mlp.mlp import RuntimePredictor
+from habitat_amd.analysis.predictor import Predictor
+from habitat_amd.analysis.wave_scaling.batch import (DeviceTable, KernelRecords, ratio_scale,
+                                                     wave_scale, wave_scale_sum)
+from oracle import lib as olib
+from oracle import mlp as omlp
+from oracle import predictor as opred
+
+pytestmark = pytest.mark.gpu
+
+
+def odev(d):
+    return oracle_device(d.as_dict())
+
+
+def oracle_sums(rec, origin, dest, segment, n_seg):
+    want = olib.wave_scale(odev(origin), odev(dest), rec)
+    sums = np.zeros(n_seg)
+    ok = want["status"] == 0
+    np.add.at(sums, segment[ok], want["time_ns"][ok])
+    return sums, int((~ok).sum())
+
+
+@pytest.mark.parametrize("n,n_seg,sorted_segments", [(1, 1, True), (63, 5, True), (64, 1, True),
+                                                     (1000, 37, True), (1000, 37, False),
+                                                     (5000, 1, True), (4097, 300, True)])
+def test_fused_sums_match_oracle(n, n_seg, sorted_segments):
+    origin = Device.V100
+    rec, _ = synthetic.kernel_records(n, origin, seed=n + n_seg, metrics_fraction=0.5)
+    rng = np.random.default_rng(n)
+    segment = rng.integers(0, n_seg, n).astype(np.int32)
+    if sorted_segments:
+        segment.sort()
+    dests = [Device.MI355X, Device.T4, Device.P100, Device.P4000, Device.V100]
+    table = DeviceTable(origin, dests)
+    sums, bad = wave_scale_sum(KernelRecords.from_numpy(rec), table,
+                               torch.from_numpy(segment).cuda(), n_seg)
+    sums, bad = sums.cpu().numpy(), bad.cpu().numpy()
+    for di, d in enumerate(dests):
+        want, want_bad = oracle_sums(rec, origin, d, segment, n_seg)
+        np.testing.assert_allclose(sums[di], want, rtol=1e-6, atol=0)
+        assert bad[di] == want_bad
+
+
+def test_fused_sums_count_records_the_reference_would_raise_on(kat):
+    base = dict(kat["scaling_record"])
+    rows = [dict(base, num_blocks=10, dynamic_smem=60000),        # status 2 on V100
+            dict(base, num_blocks=100, dram_read_bytes=-3e8),     # status 3 everywhere
+            dict(base, num_blocks=4096), dict(base, num_blocks=50)]
+    rec = {k: np.array([r[k] for r in rows]) for k in rows[0]}
+    table = DeviceTable(Device.MI355X, [Device.V100, Device.MI355X])
+    sums, bad = wave_scale_sum(KernelRecords.from_numpy(rec), table)
+    assert bad.cpu().tolist() == [2, 1]
+    for di, d in enumerate([Device.V100, Device.MI355X]):
+        want, _ = oracle_sums(rec, Device.MI355X, d, np.zeros(4, np.int32), 1)
+        np.testing.assert_allclose(sums[di].cpu().numpy(), want, rtol=1e-6)
+
+
+def test_fused_sums_equal_the_per_record_kernel_summed():
+    origin = Device.V100
+    rec, _ = synthetic.kernel_records(20_000, origin, seed=77)
+    devices, _ = synthetic.device_sweep(40, seed=1)
+    kr = KernelRecords.from_numpy(rec)
+    per_record = wave_scale(kr, origin, devices)
+    sums, bad = wave_scale_sum(kr, DeviceTable(origin, devices))
+    t = torch.where(per_record.status == 0, per_record.time_ns, torch.zeros_like(per_record.time_ns))
+    np.testing.assert_allclose(sums[:, 0].cpu().numpy(), t.sum(dim=1).cpu().numpy(), rtol=1e-10)
+    assert torch.equal(bad, (per_record.status != 0).sum(dim=1).to(torch.int32))
+
+
+def test_ratio_scale_matches_python_arithmetic():
+    rng = np.random.default_rng(5)
+    D, O = 7, 300
+    pred = rng.normal(0.05, 0.03, size=(D + 1, O)).astype(np.float32)   # some negative
+    pred[D] = np.abs(pred[D]) + 0.01
+    ms = rng.uniform(0.01, 20.0, O)
+    totals = torch.full((D,), 2.5, dtype=torch.float64, device="cuda")
+    out = ratio_scale(torch.from_numpy(pred).cuda(), torch.from_numpy(ms).cuda(), D, totals=totals)
+    out = out.cpu().numpy()
+    for d in range(D):
+        want = [opred.special_op_ms(ms[o], float(pred[d, o]), float(pred[D, o])) for o in range(O)]
+        assert np.array_equal(out[d], np.array(want))            # same fp64 operations
+        assert totals[d].item() == pytest.approx(2.5 + sum(want), rel=1e-12)
+    assert (out == 0).any()
+
+
+def test_end_to_end_256_device_sweep():
+    """BASELINE configs[4]: a ResNet-50-shaped trace against 256 destinations."""
+    origin = Device.V100
+    trace = synthetic.resnet50_trace(origin, batch=32, seed=3)
+    preds = {}
+    for kind in ("conv2d", "linear", "bmm", "lstm"):
+        torch.manual_seed(0)
+        rp = RuntimePredictor(kind, 8, 1024)
+        x, mu, sigma = synthetic.mlp_features(kind, 2048, seed=2)
+        rp.set_normalization(mu, sigma)
+        preds[kind] = rp
+    predictor = Predictor(mlp_predictors=preds)
+    devices, feats = synthetic.device_sweep(256, seed=1)
+    device_features = {d.name: list(f) for d, f in zip(devices, feats)}
+    device_features[origin.name] = [16, 900, 80, 14.028]
+    sweep = predictor.predict_trace_sweep(trace, devices, device_features)
+    totals = sweep.total_ms.cpu().numpy()
+    assert totals.shape == (256,) and np.all(np.isfinite(totals)) and np.all(totals > 0)
+    assert int(sweep.bad_records.sum().item()) == 0
+
+    # oracle, for a sample of destinations
+    from test_api_gpu import as_record
+    from habitat_amd.analysis import predictor as P
+    from habitat_amd.analysis.metrics import Metric
+    from oracle import wave_scaling as ows
+    o = odev(origin)
+    for di in (0, 100, 255):
+        d = odev(devices[di])
+        total = 0.0
+        for op in trace.operations:
+            if op.name in ("conv2d", "linear"):
+                rp = preds[op.name]
+                a = P._ARGUMENTS[op.name](op)
+                f = [a[x] for x in rp.model.features]
+                rows = np.array([f + device_features[devices[di].name],
+                                 f + device_features[origin.name]], np.float64)
+                y = omlp.forward_fp64(rp.model.state_dict(), rows, rp.mu, rp.sigma)
+                total += opred.special_op_ms(op.run_time_ms, y[0], y[1])
+                continue
+            for rt in (op.forward, op.backward):
+                if rt is None:
+                    continue
+                pk = []
+                for k in rt.kernels:
+                    try:
+                        m = tuple(k.get_metric(x) for x in (Metric.SinglePrecisionFLOPEfficiency,
+                                                            Metric.DRAMReadBytes,
+                                                            Metric.DRAMWriteBytes))
+                    except AttributeError:
+                        m = None
+                    pk.append(ows.unified(as_record(k, m), o, d, has_metrics=m is not None))
+                total += opred.wave_scaled_pass_ms(rt.run_time_ms,
+                                                   [k.run_time_ns for k in rt.kernels], pk)
+        assert totals[di] == pytest.approx(total, rel=1e-5)
+    # faster devices predict shorter iterations, on the whole: rank correlation
+    # between memory bandwidth and predicted time is clearly negative
+    bw = np.array([d.mem_bandwidth_gb for d in devices], float)
+    rank = lambda v: np.argsort(np.argsort(v))
+    assert np.corrcoef(rank(bw), rank(totals))[0, 1] < -0.3
+
+
+def test_device_table_argument_checks():
+    with pytest.raises(ValueError):
+        DeviceTable(Device.V100, [])
+    bad = DeviceProperties(name="z", **dict(Device.V100.as_dict(), base_clock_mhz=0))
+    with pytest.raises(_lib.HabitatLibraryError) as e:
+        DeviceTable(Device.V100, [Device.T4, bad])
+    assert e.value.code == _lib.HBT_ESPEC
