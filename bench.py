@@ -31,6 +31,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 BYTES_PER_RECORD = 68          # 5 x i32 + 4 x f64 read, f64 + 2 x i32 written
+# Measured L2<->fabric bytes per record (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled
+# on a copy kernel of known size; profiles/wave_scale_kernel_1M_and_64M_records.md):
+# 52.18 read + 17.00 written (the status byte is the 69th).
+TRAFFIC_BYTES_PER_RECORD = 69.18
+MLP_TRAFFIC_BYTES_PER_ROW = 33040.0  # profiles/mlp_fused_kernel_conv2d_1M_rows.md: weights re-streamed per round
 
 
 def parse():
@@ -46,6 +51,9 @@ def parse():
     ap.add_argument("--no-mlp", action="store_true")
     ap.add_argument("--no-large", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device-to-device copy (for scaling the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     return ap.parse_args()
 
 
@@ -121,6 +129,15 @@ def main():
     torch.cuda.set_device(0)
     origin, dest = Device.V100, Device.MI355X
 
+    if args.copy_calibration:
+        src = torch.ones(1 << 27, dtype=torch.float64, device="cuda")   # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
+
     # ---------------- wave scaling, configs[1] ----------------
     rec, stats = synthetic.kernel_records(args.records, origin, seed=0)
     records = KernelRecords.from_numpy(rec)
@@ -140,8 +157,11 @@ def main():
                    "records": args.records, "origin": origin.name, "dest": dest.name,
                    "seed": stats["seed"], "rejected_draws": stats["rejected"]},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "wave_scale_kernel<4>", "launch_us": launch_ms * 1e3,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": TRAFFIC_BYTES_PER_RECORD * args.records,
+                     "traffic_unit": "bytes/launch (FETCH_SIZE + WRITE_SIZE, rocprofv3, "
+                                     "copy-calibrated; see profiles/)",
+                     "kernel": "wave_scale_kernel<2, true>", "launch_us": launch_ms * 1e3,
                      "bytes_per_record": BYTES_PER_RECORD},
     }
 
@@ -211,7 +231,9 @@ def main():
                                       % (kind, args.mlp_rows, f_in)},
                "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_FP32_PEAK_TFLOPS,
                             "unit": "TFLOP/s", "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
-                            "traffic": None, "kernel": "mlp_fused_kernel",
+                            "traffic": (MLP_TRAFFIC_BYTES_PER_ROW * args.mlp_rows
+                                        if kind == "conv2d" else None),
+                            "kernel": "mlp_fused_kernel<4>",
                             "launch_ms": m_launch, "flops_per_row": flops_per_row}}
         if not args.no_cpu:
             from oracle import mlp as omlp
