@@ -113,7 +113,7 @@ def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported "
-              "(records and rows are independent and would shard by ranges, see DESIGN.md)"
+              "(records and rows are independent and would shard by contiguous ranges)"
               % args.gpus, file=sys.stderr)
         sys.exit(2)
 

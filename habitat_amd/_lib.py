@@ -77,6 +77,11 @@ def lib():
             raise ImportError(
                 "habitat_amd: %s is missing — build it with `python -m habitat_amd.build` "
                 "(there is no CPU fallback)" % LIB_PATH)
+        # The library and torch must share one HIP runtime: torch ships its own
+        # libamdhip64, and whichever copy is loaded first serves both.  Import
+        # torch first so that streams and device pointers it hands over belong
+        # to the runtime the kernels are launched on.
+        import torch  # noqa: F401
         handle = C.CDLL(LIB_PATH)
         for name, (res, args) in list(_SIGNATURES.items()) + list(_OPTIONAL.items()):
             fn = getattr(handle, name)

@@ -32,6 +32,12 @@ def register_device(name, mem, mem_bw, num_sm, single, **extra):
     DEVICE_FEATURES[name] = [row[p] for p in DEVICE_PARAMS]
 
 
+def unregister_device(name):
+    """Remove a row added with register_device."""
+    _TABLE.pop(name, None)
+    DEVICE_FEATURES.pop(name, None)
+
+
 def get_device_features(device_name, device_params):
     """[row[p] for p in device_params] of one device.  An unknown device raises
     IndexError, as the reference's pandas lookup does (devices.py:9)."""

@@ -108,6 +108,11 @@ MLP_FEATURES = {
 }
 
 
+# The six devices of the reference's MLP device table (analysis/mlp/devices.csv:2-7);
+# a fixed list, so that seeded inputs do not depend on rows registered later.
+REFERENCE_MLP_DEVICES = ("P100", "P4000", "RTX2070", "RTX2080Ti", "T4", "V100")
+
+
 def mlp_features(kind, n, seed=2, device_features=None):
     """[n, F+4] float64 raw feature rows for one MLP kind: the operation
     features in MLP_FEATURES order, then [mem, mem_bw, num_sm, single] of a
@@ -134,7 +139,7 @@ def mlp_features(kind, n, seed=2, device_features=None):
     else:
         raise KeyError(kind)
     if device_features is None:
-        device_features = np.array([DEVICE_FEATURES[k] for k in sorted(DEVICE_FEATURES)],
+        device_features = np.array([DEVICE_FEATURES[k] for k in REFERENCE_MLP_DEVICES],
                                    np.float64)
     dev = device_features[rng.integers(0, device_features.shape[0], size=n)]
     x = np.concatenate([np.stack([cols[f] for f in MLP_FEATURES[kind]], axis=1), dev], axis=1)

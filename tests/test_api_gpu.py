@@ -204,13 +204,19 @@ def test_device_sweep_matches_per_device_prediction():
     predictor = Predictor(mlp_predictors=preds)
     devices, feats = synthetic.device_sweep(24, seed=1)
     from habitat_amd.analysis.mlp import devices as md
-    for d, f in zip(devices, feats):
-        md.register_device(d.name, *f)
-    totals = trace.to_devices(devices, predictor)
-    assert len(totals) == 24
-    for i in (0, 7, 23):
-        want = trace.to_device(devices[i], predictor).run_time_ms
-        assert totals[i] == pytest.approx(want, rel=1e-9)
-    oracle_total = opred.trace_ms([oracle_operation_ms(op, devices[3], preds)
-                                   for op in trace.operations])
-    assert totals[3] == pytest.approx(oracle_total, rel=1e-5)
+    before = dict(md.DEVICE_FEATURES)
+    try:
+        for d, f in zip(devices, feats):
+            md.register_device(d.name, *f)
+        totals = trace.to_devices(devices, predictor)
+        assert len(totals) == 24
+        for i in (0, 7, 23):
+            want = trace.to_device(devices[i], predictor).run_time_ms
+            assert totals[i] == pytest.approx(want, rel=1e-9)
+        oracle_total = opred.trace_ms([oracle_operation_ms(op, devices[3], preds)
+                                       for op in trace.operations])
+        assert totals[3] == pytest.approx(oracle_total, rel=1e-5)
+    finally:
+        for d in devices:
+            md.unregister_device(d.name)
+        assert md.DEVICE_FEATURES == before
