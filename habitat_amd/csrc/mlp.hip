@@ -19,8 +19,11 @@
 //
 // Weights are repacked once, at hbt_mlp_create, so that a wave's fragment for
 // 8 consecutive k is one fully coalesced 1 KiB load (16 B per lane) straight
-// into the registers the MFMA reads: index [wave][k/8][tile][lane][4] holds
-// W[32*tile_global + lane%32][8*(k/8) + 4*(lane/32) + e].  The matching
+// into the registers the MFMA reads: index [wave][layer][k/8][tile][lane][4]
+// holds W_layer[32*tile_global + lane%32][8*(k/8) + 4*(lane/32) + e].  For one
+// wave the k-groups of all layers form one contiguous stream, so the prefetch
+// ring runs across layer boundaries: the next layer's first weights are already
+// in flight while this layer's results are written back.  The matching
 // activation fragment is one ds_read_b128 of Act[lane%32][8*(k/8) + 4*(lane/32) ..+3];
 // rows are padded by 4 floats so those reads are bank-conflict free.
 //
@@ -55,17 +58,16 @@ struct MlpArgs {
   int32_t hidden;
   const double* mu;      // [in_features]
   const double* sigma;   // [in_features]
-  const float* w_first;  // packed fc1 [waves][in_padded/8][tpw][64][4]
-  const float* w_hidden; // packed hidden layers, kWidth*kWidth floats each
+  const float* w_stream; // packed weights [waves][groups of all layers][tpw][64][4]
   const float* bias;     // [(hidden + 1)][kWidth]: fc1 bias, then hidden biases
   const float* w_last;   // fc2.weight [kWidth]
   float b_last;
 };
 
-// One layer's K loop for this wave: acc[tile] += Wfrag * Actfrag over kg groups
-// of 8 k (kg a multiple of 4).  Fragments travel through a ring of four
-// register slots: the loads for group j+3 are issued before the MFMAs of group
-// j, so a fragment has three MFMA blocks (>= 3 * 16 * TPW * 4 cycles) to arrive.
+// Fragments travel through a ring of four register slots.  Weight fragments are
+// indexed by the wave's global k-group number (all layers, one stream) and are
+// loaded three groups ahead, also across a layer boundary; activation
+// fragments are loaded from LDS three groups ahead within the layer.
 template <int TPW>
 struct Ring {
   f32x4 w[4][TPW];
@@ -73,11 +75,15 @@ struct Ring {
 };
 
 template <int TPW, int SLOT>
-__device__ __forceinline__ void ring_load(Ring<TPW>& r, const f32x4* __restrict__ wp, int g,
-                                          const float* act_lane, int lane) {
-  const f32x4* p = wp + (size_t)g * TPW * 64 + lane;
+__device__ __forceinline__ void ring_load_w(Ring<TPW>& r, const f32x4* __restrict__ stream,
+                                            int group, int lane) {
+  const f32x4* p = stream + (size_t)group * TPW * 64 + lane;
 #pragma unroll
   for (int t = 0; t < TPW; ++t) r.w[SLOT][t] = p[t * 64];
+}
+
+template <int TPW, int SLOT>
+__device__ __forceinline__ void ring_load_x(Ring<TPW>& r, const float* act_lane, int g) {
   r.x[SLOT] = *reinterpret_cast<const f32x4*>(act_lane + 8 * g);
 }
 
@@ -90,32 +96,40 @@ __device__ __forceinline__ void ring_mfma(const Ring<TPW>& r, f32x16 (&acc)[TPW]
       acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(r.w[SLOT][t][e], r.x[SLOT][e], acc[t], 0, 0, 0);
 }
 
+// One layer's K loop: kg groups of 8 k (a multiple of 4) starting at global
+// group `g0` of the wave's stream; `g_end` is the stream's last valid group.
+// On entry ring slots 0..2 hold the weights of groups g0..g0+2.
 template <int TPW>
-__device__ __forceinline__ void layer_k_loop(const f32x4* __restrict__ wp, int kg,
-                                             const float* act_lane, f32x16 (&acc)[TPW]) {
+__device__ __forceinline__ void layer_k_loop(Ring<TPW>& r, const f32x4* __restrict__ stream,
+                                             int g0, int kg, int g_end, const float* act_lane,
+                                             f32x16 (&acc)[TPW]) {
   const int lane = threadIdx.x & 63;
   const int last = kg - 1;
-  Ring<TPW> r;
-  ring_load<TPW, 0>(r, wp, 0, act_lane, lane);
-  ring_load<TPW, 1>(r, wp, 1, act_lane, lane);
-  ring_load<TPW, 2>(r, wp, 2, act_lane, lane);
+  ring_load_x<TPW, 0>(r, act_lane, 0);
+  ring_load_x<TPW, 1>(r, act_lane, min(1, last));
+  ring_load_x<TPW, 2>(r, act_lane, min(2, last));
   for (int j = 0; j < kg; j += 4) {
     // The scheduling barriers keep the compiler from sinking a prefetch below
-    // the MFMA block it is meant to overlap with.  Groups past the end reload
-    // the last one (valid memory, unused values).
-    ring_load<TPW, 3>(r, wp, min(j + 3, last), act_lane, lane);
+    // the MFMA block it is meant to overlap with.  Weight groups past the end
+    // of the stream, and activation groups past the end of the layer, reload
+    // the last valid one (unused values).
+    ring_load_w<TPW, 3>(r, stream, min(g0 + j + 3, g_end), lane);
+    ring_load_x<TPW, 3>(r, act_lane, min(j + 3, last));
     __builtin_amdgcn_sched_barrier(0);
     ring_mfma<TPW, 0>(r, acc);
     __builtin_amdgcn_sched_barrier(0);
-    ring_load<TPW, 0>(r, wp, min(j + 4, last), act_lane, lane);
+    ring_load_w<TPW, 0>(r, stream, min(g0 + j + 4, g_end), lane);
+    ring_load_x<TPW, 0>(r, act_lane, min(j + 4, last));
     __builtin_amdgcn_sched_barrier(0);
     ring_mfma<TPW, 1>(r, acc);
     __builtin_amdgcn_sched_barrier(0);
-    ring_load<TPW, 1>(r, wp, min(j + 5, last), act_lane, lane);
+    ring_load_w<TPW, 1>(r, stream, min(g0 + j + 5, g_end), lane);
+    ring_load_x<TPW, 1>(r, act_lane, min(j + 5, last));
     __builtin_amdgcn_sched_barrier(0);
     ring_mfma<TPW, 2>(r, acc);
     __builtin_amdgcn_sched_barrier(0);
-    ring_load<TPW, 2>(r, wp, min(j + 6, last), act_lane, lane);
+    ring_load_w<TPW, 2>(r, stream, min(g0 + j + 6, g_end), lane);
+    ring_load_x<TPW, 2>(r, act_lane, min(j + 6, last));
     __builtin_amdgcn_sched_barrier(0);
     ring_mfma<TPW, 3>(r, acc);
     __builtin_amdgcn_sched_barrier(0);
@@ -150,7 +164,19 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
   const float* act_lane = act + m * kStride + 4 * h;
   const int tile0 = wave * TPW;  // first n-tile of this wave
 
+  // This wave's weight stream: fc1's groups, then 128 groups per hidden layer.
+  const int kg_first = a.in_padded / 8;
+  const int groups = kg_first + a.hidden * (kWidth / 8);
+  const f32x4* stream = reinterpret_cast<const f32x4*>(a.w_stream) + (size_t)wave * groups * TPW * 64;
+  const int g_end = groups - 1;
+
+  Ring<TPW> ring;
+  ring_load_w<TPW, 0>(ring, stream, 0, lane);
+  ring_load_w<TPW, 1>(ring, stream, min(1, g_end), lane);
+  ring_load_w<TPW, 2>(ring, stream, min(2, g_end), lane);
+
   f32x16 acc[TPW];
+  int g0 = 0;
   for (int layer = 0; layer <= a.hidden; ++layer) {
     // accumulators start at the bias of their output column
     const float* bias = a.bias + (size_t)layer * kWidth;
@@ -163,16 +189,9 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
         for (int e = 0; e < 4; ++e) acc[t][4 * g + e] = b[e];
       }
 
-    if (layer == 0) {
-      const int kg = a.in_padded / 8;
-      const f32x4* wp = reinterpret_cast<const f32x4*>(a.w_first) + (size_t)wave * kg * TPW * 64;
-      layer_k_loop<TPW>(wp, kg, act_lane, acc);
-    } else {
-      constexpr int kg = kWidth / 8;
-      const f32x4* wp = reinterpret_cast<const f32x4*>(a.w_hidden) +
-                        ((size_t)(layer - 1) * WAVES + wave) * kg * TPW * 64;
-      layer_k_loop<TPW>(wp, kg, act_lane, acc);
-    }
+    const int kg = (layer == 0) ? kg_first : kWidth / 8;
+    layer_k_loop<TPW>(ring, stream, g0, kg, g_end, act_lane, acc);
+    g0 += kg;
 
     __syncthreads();  // every wave has finished reading this layer's input
 #pragma unroll
@@ -228,8 +247,7 @@ struct hbt_mlp {
   void* blob;          // one device allocation holding everything below
   const double* mu;
   const double* sigma;
-  const float* w_first;
-  const float* w_hidden;
+  const float* w_stream;
   const float* bias;
   const float* w_last;
   float b_last;
@@ -238,9 +256,10 @@ struct hbt_mlp {
 namespace hbt {
 namespace {
 
-// Repack a row-major [kWidth][k_in] weight matrix (k_in <= k_padded) into
-// [waves][k_padded/8][tpw][64 lanes][4].
-void pack_layer(const float* W, int k_in, int k_padded, int waves, float* dst) {
+// Repack one layer, a row-major [kWidth][k_in] weight matrix (k_in <= k_padded),
+// into the per-wave streams: wave w's copy goes to dst + w * wave_stride as
+// [k_padded/8][tpw][64 lanes][4].
+void pack_layer(const float* W, int k_in, int k_padded, int waves, float* dst, size_t wave_stride) {
   const int tpw = (kWidth / 32) / waves;
   const int kg = k_padded / 8;
   for (int w = 0; w < waves; ++w)
@@ -251,7 +270,7 @@ void pack_layer(const float* W, int k_in, int k_padded, int waves, float* dst) {
             const int n = (w * tpw + t) * 32 + (lane & 31);
             const int k = 8 * j + 4 * (lane >> 5) + e;
             const float v = (k < k_in) ? W[(size_t)n * k_in + k] : 0.f;
-            dst[((((size_t)w * kg + j) * tpw + t) * 64 + lane) * 4 + e] = v;
+            dst[(size_t)w * wave_stride + (((size_t)j * tpw + t) * 64 + lane) * 4 + e] = v;
           }
 }
 
@@ -289,14 +308,16 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
   }
 
   // Host image of the device blob.
-  const size_t n_first = (size_t)kWidth * in_padded;
-  const size_t n_hidden = (size_t)hidden_layers * kWidth * kWidth;
+  // floats per wave: (fc1 groups + 128 per hidden layer) x tpw x 64 lanes x 4
+  const int tpw = (kWidth / 32) / kWaves;
+  const size_t group_floats = (size_t)tpw * 64 * 4;
+  const size_t wave_stride = ((size_t)in_padded / 8 + (size_t)hidden_layers * (kWidth / 8)) * group_floats;
+  const size_t n_stream = wave_stride * kWaves;
   const size_t n_bias = (size_t)(hidden_layers + 1) * kWidth;
   size_t off = 0;
   const size_t off_mu = off; off = align_up(off + sizeof(double) * in_features, 256);
   const size_t off_sigma = off; off = align_up(off + sizeof(double) * in_features, 256);
-  const size_t off_first = off; off = align_up(off + sizeof(float) * n_first, 256);
-  const size_t off_hidden = off; off = align_up(off + sizeof(float) * n_hidden, 256);
+  const size_t off_stream = off; off = align_up(off + sizeof(float) * n_stream, 256);
   const size_t off_bias = off; off = align_up(off + sizeof(float) * n_bias, 256);
   const size_t off_last = off; off = align_up(off + sizeof(float) * kWidth, 256);
   const size_t total = off;
@@ -310,10 +331,11 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
   }
   std::memcpy(host.data() + off_mu, mu, sizeof(double) * in_features);
   std::memcpy(host.data() + off_sigma, sigma, sizeof(double) * in_features);
-  pack_layer(W[0], in_features, in_padded, kWaves, reinterpret_cast<float*>(host.data() + off_first));
+  float* stream = reinterpret_cast<float*>(host.data() + off_stream);
+  pack_layer(W[0], in_features, in_padded, kWaves, stream, wave_stride);
   for (int l = 0; l < hidden_layers; ++l)
     pack_layer(W[1 + l], kWidth, kWidth, kWaves,
-               reinterpret_cast<float*>(host.data() + off_hidden) + (size_t)l * kWidth * kWidth);
+               stream + ((size_t)in_padded / 8 + (size_t)l * (kWidth / 8)) * group_floats, wave_stride);
   for (int l = 0; l <= hidden_layers; ++l)
     std::memcpy(host.data() + off_bias + sizeof(float) * (size_t)l * kWidth, b[l],
                 sizeof(float) * kWidth);
@@ -355,8 +377,7 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
   m->blob = blob;
   m->mu = reinterpret_cast<const double*>(base + off_mu);
   m->sigma = reinterpret_cast<const double*>(base + off_sigma);
-  m->w_first = reinterpret_cast<const float*>(base + off_first);
-  m->w_hidden = reinterpret_cast<const float*>(base + off_hidden);
+  m->w_stream = reinterpret_cast<const float*>(base + off_stream);
   m->bias = reinterpret_cast<const float*>(base + off_bias);
   m->w_last = reinterpret_cast<const float*>(base + off_last);
   m->b_last = b[hidden_layers + 1][0];
@@ -390,8 +411,7 @@ int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* 
   a.hidden = mlp->hidden;
   a.mu = mlp->mu;
   a.sigma = mlp->sigma;
-  a.w_first = mlp->w_first;
-  a.w_hidden = mlp->w_hidden;
+  a.w_stream = mlp->w_stream;
   a.bias = mlp->bias;
   a.w_last = mlp->w_last;
   a.b_last = mlp->b_last;
