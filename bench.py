@@ -51,6 +51,10 @@ def parse():
     ap.add_argument("--no-mlp", action="store_true")
     ap.add_argument("--no-large", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-ceilings", action="store_true",
+                    help="skip measuring the box's own copy bandwidth and FMA/MFMA rates")
+    ap.add_argument("--mlp-other-kinds", default="linear,bmm,lstm",
+                    help="further MLP kinds timed with one step each (empty to skip)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy (for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -248,7 +252,33 @@ def main():
                 "value": m / dt, "unit": "rows/s", "cores": threads, "kind": "port",
                 "sample": "oracle/mlp.py forward_fp32 (torch CPU fp32, one batched forward) on "
                           "the first %d rows, %d torch threads" % (m, threads)}
+        others = {}
+        for other in [k for k in args.mlp_other_kinds.split(",") if k and k != kind]:
+            torch.manual_seed(0)
+            rpo = RuntimePredictor(other, 8, 1024)
+            xo, muo, sgo = synthetic.mlp_features(other, args.mlp_rows, seed=2)
+            rpo.set_normalization(muo, sgo)
+            xog = torch.from_numpy(xo).cuda()
+            _, o_launch = time_steps(lambda: rpo.predict_batch(xog, out=yg), 1, 1)
+            fl = 2.0 * (xo.shape[1] * 1024 + 8 * 1024 * 1024 + 1024)
+            tf = fl * args.mlp_rows / (o_launch * 1e-3) / 1e12
+            others[other] = {"rows": args.mlp_rows, "launch_ms": o_launch,
+                             "value": args.mlp_rows / (o_launch * 1e-3), "unit": "rows/s",
+                             "achieved": tf, "frac": tf / MFMA_FP32_PEAK_TFLOPS}
+            del rpo, xog
+        if others:
+            mlp["other_kinds"] = others
         result["mlp"] = mlp
+
+    # ---------------- what this box itself can do (ceilings under the published peaks) ----------
+    if not args.no_ceilings:
+        from habitat_amd import device_info
+        name, _ = device_info.local_device(0)
+        m = device_info.measure()
+        result["measured_ceilings"] = {
+            "device": name, "copy_GBps_read_plus_write": m["copy_gbps"],
+            "fp32_mfma_TFLOPs": m["fp32_mfma_gflops"] / 1e3,
+            "fp32_vector_fma_TFLOPs": m["fp32_fma_gflops"] / 1e3}
 
     print(json.dumps(result))
 

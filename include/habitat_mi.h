@@ -214,6 +214,29 @@ int hbt_mlp_forward(hbt_mlp *mlp, const double *raw_features, int64_t n, float *
                     void *hip_stream);
 void hbt_mlp_destroy(hbt_mlp *mlp);
 
+/*
+ * Calibration of the GPU this process runs on.  Not part of the prediction
+ * path: these calls allocate their own scratch memory, use the default stream
+ * and synchronise.
+ *
+ * hbt_local_device_spec fills `out` (host) from hipDeviceProp_t, the fields the
+ * reference's device_info tool prints from cudaDeviceProp
+ * (cpp/src/device_info.cpp:16-30), plus bandwidth, clock and vector-fp32 peak
+ * derived from the reported clocks; `name` (host, nullable) receives the device
+ * name.  The compute capability is HIP's, so the spec is a description, not an
+ * input the occupancy model accepts as is.
+ *
+ * hbt_measure_fp32_fma_gflops times a kernel of independent fp32 FMAs, the
+ * role of the reference's flop_test kernel (cpp/src/cuda/diagnostics.cu:9-25,
+ * tools/device-metadata/measure_peak_flops.py:10-18); hbt_measure_fp32_mfma_gflops
+ * does the same with v_mfma_f32_32x32x2_f32; hbt_measure_copy_gbps times a
+ * device-to-device copy of `bytes` (read + write counted).
+ */
+int hbt_local_device_spec(int device, hbt_device_spec *out, char *name, size_t name_len);
+int hbt_measure_fp32_fma_gflops(int iters, double *out_gflops);
+int hbt_measure_fp32_mfma_gflops(int iters, double *out_gflops);
+int hbt_measure_copy_gbps(size_t bytes, double *out_gbps);
+
 #ifdef __cplusplus
 }
 #endif

@@ -220,3 +220,18 @@ def test_device_sweep_matches_per_device_prediction():
         for d in devices:
             md.unregister_device(d.name)
         assert md.DEVICE_FEATURES == before
+
+
+def test_local_device_description_and_measured_ceilings():
+    from habitat_amd import device_info
+    name, props = device_info.local_device(0)
+    assert isinstance(name, str) and len(name) > 0
+    assert props["warp_size"] == 64 and props["num_sms"] >= 1
+    assert props["max_threads_per_block"] == 1024 and props["shared_mem_per_block"] >= 65536
+    from habitat_amd import DeviceProperties
+    dev = DeviceProperties(name="local", **props)        # the keys are DeviceProperties' own
+    assert dev.num_sms == props["num_sms"]
+    m = device_info.measure(iters=2000, copy_bytes=1 << 28)
+    # an MI355X: several TB/s of copy bandwidth, tens of TFLOP/s of fp32
+    assert m["copy_gbps"] > 500 and m["fp32_fma_gflops"] > 5000 and m["fp32_mfma_gflops"] > 20000
+    assert m["fp32_mfma_gflops"] > m["fp32_fma_gflops"]

@@ -237,3 +237,25 @@ def test_metadata_manager_sqlite(tmp_path):
     assert mm.kernel_registers_for(gemm, Device.T4) == 128        # 70 <= 75
     assert mm.kernel_registers_for(relu, Device.V100) is None     # only a newer arch listed
     assert mm.registers_for_names(["gemm", "relu", "x"], Device.T4) == [128, 16, -1]
+
+
+def test_csv_reports(tmp_path):
+    import csv
+    from habitat_amd.analysis import report
+    from habitat_amd.analysis.arguments import Arguments
+    from habitat_amd.analysis.operation import MeasuredOperation
+    from habitat_amd.analysis.run_time import RunTimeMeasurement
+    from habitat_amd.analysis.trace import Trace
+    v100 = Device.V100
+    ops = [MeasuredOperation("relu_", Arguments((), {}), RunTimeMeasurement(1.5, [], v100),
+                             RunTimeMeasurement(0.25, [], v100), v100),
+           MeasuredOperation("conv2d", Arguments((), {}), RunTimeMeasurement(4.0, [], v100), None, v100)]
+    trace = Trace(v100, ops)
+    assert trace.run_time_ms == 5.75
+    p = report.record_breakdown("resnet50+16", v100, Device.T4, trace, str(tmp_path))
+    assert p.endswith("resnet50+16-V100-T4-breakdown.csv")
+    assert list(csv.reader(open(p))) == [["operation", "run_time_ms"], ["relu_", "1.75"], ["conv2d", "4.0"]]
+    p = report.record_sweep("resnet50+16", trace, [Device.T4, Device.P100], [9.5, 7.25], str(tmp_path))
+    assert p.endswith("resnet50+16-V100-e2e.csv")
+    assert list(csv.reader(open(p))) == [["device", "run_time_ms"], ["V100", "5.75"], ["T4", "9.5"],
+                                         ["P100", "7.25"]]
