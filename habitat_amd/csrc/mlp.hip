@@ -14,8 +14,8 @@
 // B operand a 2(k) x 32(m) activation fragment.  The 32 n-tiles of a layer are
 // split over the waves; a wave keeps its slice of the output in accumulator
 // registers for the whole K loop and only then, after a barrier, overwrites the
-// LDS activations in place (bias enters as the accumulator's initial value,
-// ReLU is applied on the way out).
+// LDS activations in place (bias, staged in LDS during the K loop, and ReLU are
+// applied on the way out).
 //
 // Weights are repacked once, at hbt_mlp_create, so that a wave's fragment for
 // 8 consecutive k is one fully coalesced 1 KiB load (16 B per lane) straight
@@ -143,6 +143,8 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* act = lds;                           // [kRows][kStride]
   float* red = lds + kRows * kStride;         // [THREADS / 32][32]
+  float* bias_lds = red + (THREADS / 32) * 32;  // [kWidth]
+  static_assert(THREADS * 4 == kWidth, "one float4 of bias per thread");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -178,30 +180,32 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
   f32x16 acc[TPW];
   int g0 = 0;
   for (int layer = 0; layer <= a.hidden; ++layer) {
-    // accumulators start at the bias of their output column
-    const float* bias = a.bias + (size_t)layer * kWidth;
+    // This layer's bias goes through LDS: every thread fetches four values now
+    // and parks them in LDS after the K loop, so that the write-back below
+    // finds them without waiting for global memory.
+    const f32x4 bias_part =
+        *reinterpret_cast<const f32x4*>(a.bias + (size_t)layer * kWidth + 4 * tid);
 #pragma unroll
     for (int t = 0; t < TPW; ++t)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x4 b = *reinterpret_cast<const f32x4*>(bias + (tile0 + t) * 32 + 8 * g + 4 * h);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[t][4 * g + e] = b[e];
-      }
+      for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
 
     const int kg = (layer == 0) ? kg_first : kWidth / 8;
     layer_k_loop<TPW>(ring, stream, g0, kg, g_end, act_lane, acc);
     g0 += kg;
 
+    *reinterpret_cast<f32x4*>(bias_lds + 4 * tid) = bias_part;
     __syncthreads();  // every wave has finished reading this layer's input
 #pragma unroll
     for (int t = 0; t < TPW; ++t)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        const int n = (tile0 + t) * 32 + 8 * g + 4 * h;
+        const f32x4 b = *reinterpret_cast<const f32x4*>(bias_lds + n);
         f32x4 o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = fmaxf(acc[t][4 * g + e], 0.f);
-        *reinterpret_cast<f32x4*>(act + m * kStride + (tile0 + t) * 32 + 8 * g + 4 * h) = o;
+        for (int e = 0; e < 4; ++e) o[e] = fmaxf(acc[t][4 * g + e] + b[e], 0.f);
+        *reinterpret_cast<f32x4*>(act + m * kStride + n) = o;
       }
     __syncthreads();
   }
@@ -235,7 +239,8 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
 }
 
 constexpr int kWaves = 4;  // one wave per SIMD: measured faster than two (fewer, longer MFMA runs between load bursts)
-constexpr size_t kLdsBytes = (size_t)(kRows * kStride + (kWaves * 64 / 32) * 32) * sizeof(float);
+constexpr size_t kLdsBytes =
+    (size_t)(kRows * kStride + (kWaves * 64 / 32) * 32 + kWidth) * sizeof(float);
 
 }  // namespace
 
