@@ -27,10 +27,10 @@ DestArgs make_dest_args(const hbt_device_spec& o, const hbt_device_spec& d) {
   p.ridge = d.peak_gflops / d.mem_bandwidth_gb;
   p.half_ridge = 0.5 * p.ridge;
   p.neg_half_over_ridge = -0.5 / p.ridge;
-  p.bw_ratio = o.mem_bandwidth_gb / d.mem_bandwidth_gb;
+  const double bw_ratio = o.mem_bandwidth_gb / d.mem_bandwidth_gb;
   const double clk_ratio = o.base_clock_mhz / d.base_clock_mhz;
   const double sm_ratio = (double)o.num_sms / (double)d.num_sms;
-  p.log2_bw = std::log2(p.bw_ratio);
+  p.log2_bw = std::log2(bw_ratio);
   p.log2_clk = std::log2(clk_ratio);
   p.log2_clk_sm = p.log2_clk + std::log2(sm_ratio);
   return p;

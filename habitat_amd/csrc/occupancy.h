@@ -16,7 +16,7 @@
 // three divisions.  Two implementations of that part: occupancy_core in 64-bit
 // arithmetic with plain C division (host, and the kernel variant for devices
 // with huge limits), and occupancy_fast in 32-bit arithmetic with a
-// float-reciprocal division that is exact for operands below 2^22 (the kernel's
+// float-reciprocal division that is exact for operands below 2^20 (the kernel's
 // normal path, taken when every device constant is small enough — which every
 // real device is).
 #pragma once
@@ -37,7 +37,7 @@ namespace hbt {
 // OccDevice::flags
 enum : uint32_t {
   kOk = 1u << 0,         // the model accepts this device (else occupancy 0 everywhere)
-  kFastOk = 1u << 1,     // every constant is small enough for occupancy_fast
+  kFastOk = 1u << 1,     // every constant is below 2^20: occupancy_fast applies
   kGp100 = 1u << 2,      // cc 6.0: 2 sub-partitions, re-checked with 4
   kVolta = 1u << 3,      // cc 7.0/7.2: pool steps 0/8/16/32/64 KB/all
   kTuring = 1u << 4,     // cc 7.5: pool steps 32 KB/all
@@ -115,7 +115,8 @@ inline OccDevice make_occ_device(const hbt_device_spec& s) {
   if (pow2) flags |= kWarpPow2;
   d.pref_pool = (major == 7) ? volta_pool(flags, d.smem_per_sm, d.smem_per_sm) : d.smem_per_sm;
   if (major == 7 && d.pref_pool < d.smem_per_block) flags |= kPoolSteps;
-  const int32_t lim = 1 << 22;
+  // every division operand below 2^20 (so that dividend + divisor <= 2^21)
+  const int32_t lim = 1 << 20;
   const bool fast = !ok ||  // a rejected device needs no arithmetic at all
                     (d.warp_size <= 1024 && d.max_threads_per_block < lim - 1024 &&
                      d.max_warps_per_sm < lim && d.regs_per_subpart < lim &&
@@ -126,11 +127,13 @@ inline OccDevice make_occ_device(const hbt_device_spec& s) {
   return d;
 }
 
-// Exact a / b for 0 <= a < 2^22, 0 < b < 2^24, given rb = 1 / float(b) to within
-// 1 ulp.  float(a) and float(b) are exact and the product rounds once more, so
-// the truncated estimate is within 1 of the quotient; one correction step in
-// each direction makes it exact.  On the host (used to test the 32-bit model)
-// it is plain division.
+// Exact a / b for a >= 0, b > 0 and a + b <= 2^21, given rb = 1 / float(b) to
+// within 1 ulp: floor((a + 1/2) * rb) in float arithmetic.  (a + 1/2) / b lies
+// in [k + 1/(2b), k + 1 - 1/(2b)] for the quotient k; the computed value is off
+// by a relative 1.5 * 2^-23 at most (reciprocal within an ulp, one rounding of
+// the product), i.e. by less than (k + 1) * 1.5 * 2^-23 <= 1/(2b) as long as
+// (k + 1) * b <= a + b <= 2^21, so truncation gives k with no correction step.
+// On the host (used to test the 32-bit model) it is plain division.
 HBT_HD float fast_rcp(int32_t b) {
 #if defined(__HIP_DEVICE_COMPILE__)
   return __builtin_amdgcn_rcpf(__int2float_rn(b));
@@ -141,11 +144,8 @@ HBT_HD float fast_rcp(int32_t b) {
 
 HBT_HD int32_t fast_div_r(int32_t a, int32_t b, float rb) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  int32_t q = (int32_t)(__int2float_rn(a) * rb);
-  const int32_t r = a - __mul24(q, b);  // q, b < 2^24 and the product fits 32 bits
-  q += (r >= b) ? 1 : 0;
-  q -= (r < 0) ? 1 : 0;
-  return q;
+  (void)b;
+  return (int32_t)((__int2float_rn(a) + 0.5f) * rb);
 #else
   (void)rb;
   return a / b;
@@ -173,8 +173,8 @@ HBT_HD int32_t smem_sum(int32_t static_smem, int32_t dynamic_smem) {
 // The rounding is C division (truncating) and the rounded size is compared as
 // an unsigned 64-bit value: (total + 255) / 256 is 0 for total in -510..0
 // (nothing allocated) and negative, hence enormous, below that.  A sum the
-// 32-bit model cannot hold (enormous, or 2^22 and more) is represented by an
-// allocation of 2^22 bytes, which exceeds the per-block limit of every fast_ok
+// 32-bit model cannot hold (enormous, or 2^20 and more) is represented by an
+// allocation of 2^20 bytes, which exceeds the per-block limit of every fast_ok
 // device and so gives occupancy 0 there, as the true value would.
 struct SmemAlloc {
   int32_t alloc;  // rounded allocation in bytes
@@ -183,15 +183,15 @@ struct SmemAlloc {
 
 HBT_HD SmemAlloc smem_alloc(int32_t smem_total) {
   SmemAlloc s;
-  const bool representable = smem_total >= -510 && smem_total < (1 << 22);
+  const bool representable = smem_total >= -510 && smem_total < (1 << 20) - 255;
   const int32_t t = smem_total > 0 ? smem_total : 0;
-  s.alloc = representable ? ((t + 255) & ~255) : (1 << 22);
+  s.alloc = representable ? ((t + 255) & ~255) : (1 << 20);
   s.rcp = fast_rcp(s.alloc > 0 ? s.alloc : 1);
   return s;
 }
 
 // The occupancy model in 32-bit arithmetic, for devices with kFastOk (every
-// device constant below 2^22, warp size <= 1024).  Any int32 record is
+// device constant below 2^20, warp size <= 1024).  Any int32 record is
 // accepted: fields outside the range the divisions are exact for have
 // closed-form answers on such a device.  `regs` is already narrowed to 16 bits.
 //
@@ -203,7 +203,7 @@ HBT_HD SmemAlloc smem_alloc(int32_t smem_total) {
 HBT_HD int32_t occupancy_fast(const OccDevice& d, int32_t block, const SmemAlloc& sm,
                               int32_t regs) {
   if (!d.ok()) return 0;
-  // regs <= 256 is the per-thread limit; it also keeps regs * warp_size below 2^22
+  // regs <= 256 is the per-thread limit; it also keeps regs * warp_size below 2^19
   const bool in_range = block > 0 && block <= d.max_threads_per_block && regs <= 256;
   block = in_range ? block : 1;
   regs = in_range ? regs : 0;

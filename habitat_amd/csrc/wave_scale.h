@@ -20,8 +20,7 @@ struct DestArgs {
   double ridge;                // peak_gflops / mem_bandwidth_gb
   double half_ridge;           // 0.5 * ridge
   double neg_half_over_ridge;  // -0.5 / ridge
-  double bw_ratio;             // origin.mem_bandwidth_gb / dest.mem_bandwidth_gb
-  double log2_bw;              // log2(bw_ratio)
+  double log2_bw;              // log2(origin.mem_bandwidth_gb / dest.mem_bandwidth_gb)
   double log2_clk;             // log2(origin.base_clock_mhz / dest.base_clock_mhz)
   double log2_clk_sm;          // log2_clk + log2(origin.num_sms / dest.num_sms)
   float inv_sms;               // 1 / num_sms rounded to float

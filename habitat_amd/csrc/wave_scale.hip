@@ -38,26 +38,31 @@ constexpr int kBlock = 256;
 template <class T, int N>
 struct alignas(sizeof(T) * N) Pack { T v[N]; };
 
-// R consecutive elements starting at i, all in range: one vector access.
-template <class T, int R>
-__device__ __forceinline__ void load_r(const T* __restrict__ p, int64_t i, T (&out)[R]) {
-  const Pack<T, R> v = *reinterpret_cast<const Pack<T, R>*>(p + i);
+// R consecutive elements starting at element i, all in range: one vector
+// access.  Index is uint32_t when every byte offset of the launch fits 32 bits
+// (the address is then a uniform 64-bit base plus a 32-bit lane offset, which
+// costs no 64-bit vector arithmetic), else uint64_t.
+template <class T, int R, class Index>
+__device__ __forceinline__ void load_r(const T* __restrict__ p, Index i, T (&out)[R]) {
+  const Index byte = i * (Index)sizeof(T);
+  const Pack<T, R> v =
+      *reinterpret_cast<const Pack<T, R>*>(reinterpret_cast<const char*>(p) + (size_t)byte);
 #pragma unroll
   for (int k = 0; k < R; ++k) out[k] = v.v[k];
 }
 
-template <class T, int R>
-__device__ __forceinline__ void store_r(T* __restrict__ p, int64_t i, const T (&in)[R]) {
+template <class T, int R, class Index>
+__device__ __forceinline__ void store_r(T* __restrict__ p, Index i, const T (&in)[R]) {
   Pack<T, R> v;
 #pragma unroll
   for (int k = 0; k < R; ++k) v.v[k] = in[k];
-  *reinterpret_cast<Pack<T, R>*>(p + i) = v;
+  const Index byte = i * (Index)sizeof(T);
+  *reinterpret_cast<Pack<T, R>*>(reinterpret_cast<char*>(p) + (size_t)byte) = v;
 }
 
 // Records i .. i+R-1 (all below n) for every destination of the launch.
-template <int R, bool FAST, bool PERMUTE>
-__device__ __forceinline__ void process(const WaveScaleArgs& a, int64_t i) {
-  const int64_t n = a.n;
+template <int R, bool FAST, bool PERMUTE, class Index>
+__device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
   const double log2_lane = PERMUTE ? kLog2Int[threadIdx.x & 63] : 0.0;
   int32_t nb[R], block[R], dyn[R], stat[R], regs[R], dregs[R];
   uint8_t hm[R];
@@ -103,7 +108,7 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, int64_t i) {
 
   for (int d = 0; d < a.n_dest; ++d) {
     const DestArgs& p = a.dest[d];
-    const int64_t at = (int64_t)d * n + i;
+    const int64_t row = (int64_t)d * a.n;  // uniform: goes into the base pointer
     double ot[R];
     int32_t occ_d[R], wave_d[R];
     uint8_t st[R];
@@ -112,35 +117,44 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, int64_t i) {
       const RecordOut o = dest_part<FAST, PERMUTE>(p, rin[k], mid[k], log2_lane);
       ot[k] = o.t; occ_d[k] = o.occ_d; wave_d[k] = o.wave_d; st[k] = o.status;
     }
-    store_r<double, R>(a.out_time_ns, at, ot);
-    if (a.out_occ_dest != nullptr) store_r<int32_t, R>(a.out_occ_dest, at, occ_d);
-    if (a.out_wave_dest != nullptr) store_r<int32_t, R>(a.out_wave_dest, at, wave_d);
-    if (a.out_status != nullptr) store_r<uint8_t, R>(a.out_status, at, st);
+    store_r<double, R>(a.out_time_ns + row, i, ot);
+    if (a.out_occ_dest != nullptr) store_r<int32_t, R>(a.out_occ_dest + row, i, occ_d);
+    if (a.out_wave_dest != nullptr) store_r<int32_t, R>(a.out_wave_dest + row, i, wave_d);
+    if (a.out_status != nullptr) store_r<uint8_t, R>(a.out_status + row, i, st);
   }
 }
 
-template <int R, bool FAST>
+template <int R, bool FAST, class Index>
 __global__ __launch_bounds__(kBlock) void wave_scale_kernel(const WaveScaleArgs a) {
-  const int64_t thread = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int64_t i = thread * R;
+  const Index thread = (Index)blockIdx.x * kBlock + threadIdx.x;
+  const Index i = thread * R;
+  const Index n = (Index)a.n;
   // A wavefront whose 64 * R records are all in range takes the vector path
   // with every lane active; the last, partial wavefront of the batch goes one
   // record at a time.
-  const int64_t wave_end = ((thread | 63) + 1) * R;
-  if (wave_end <= a.n) {
-    process<R, FAST, true>(a, i);
+  const Index wave_end = ((thread | 63) + 1) * R;
+  if (wave_end <= n) {
+    process<R, FAST, true, Index>(a, i);
   } else {
-    const int64_t end = (i + R < a.n) ? i + R : a.n;
-    for (int64_t j = i; j < end; ++j) process<1, FAST, false>(a, j);
+    const Index end = (i + R < n) ? i + R : n;
+    for (Index j = i; j < end; ++j) process<1, FAST, false, Index>(a, j);
   }
+}
+
+template <int R, bool FAST, class Index>
+void launch(const WaveScaleArgs& args, hipStream_t stream) {
+  const int64_t threads = (args.n + R - 1) / R;
+  const int64_t blocks = (threads + kBlock - 1) / kBlock;
+  hipLaunchKernelGGL((wave_scale_kernel<R, FAST, Index>), dim3((unsigned)blocks), dim3(kBlock), 0,
+                     stream, args);
 }
 
 template <int R, bool FAST>
 void launch(const WaveScaleArgs& args, hipStream_t stream) {
-  const int64_t threads = (args.n + R - 1) / R;
-  const int64_t blocks = (threads + kBlock - 1) / kBlock;
-  hipLaunchKernelGGL((wave_scale_kernel<R, FAST>), dim3((unsigned)blocks), dim3(kBlock), 0, stream,
-                     args);
+  // 32-bit byte offsets when the widest column (8 bytes per record) and the
+  // thread numbering stay below 2^32 with room for the last wavefront.
+  if (args.n < ((int64_t)1 << 28)) launch<R, FAST, uint32_t>(args, stream);
+  else launch<R, FAST, uint64_t>(args, stream);
 }
 
 }  // namespace

@@ -83,8 +83,9 @@ __device__ __forceinline__ double exp2_poly(double x) {
 template <class C>
 __device__ __forceinline__ double div_const(double x) {
   constexpr double c = C::value, rc = 1.0 / C::value;
+  // safe: zero, or finite with |x| >= 2^-900 (c > 1, so nothing can overflow)
   const double ax = fabs(x);
-  if (__builtin_expect((ax > 0x1p+900) || (ax < 0x1p-900 && ax != 0.0), 0)) return x / c;
+  if (__builtin_expect(!((ax >= 0x1p-900 && ax < __builtin_inf()) || ax == 0.0), 0)) return x / c;
   const double q = x * rc;
   const double r = fma(-q, c, x);
   return fma(r, rc, q);
@@ -94,7 +95,7 @@ struct C1e9 { static constexpr double value = 1e9; };
 
 // FAST: every device of the launch has OccDevice::fast_ok, so the 32-bit model
 // applies to every record.  Otherwise the 64-bit model with real divisions runs
-// (devices with limits of 2^22 and more: not real hardware, but in the domain).
+// (devices with limits of 2^20 and more: not real hardware, but in the domain).
 template <bool FAST>
 __device__ __forceinline__ int32_t occupancy_dev(const OccDevice& d, int32_t block,
                                                  int32_t smem_total, const SmemAlloc& sm,
@@ -168,8 +169,11 @@ __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn
                    (above ? m.num_gflops : m.total_gb);
   double gamma = above ? q : p.neg_half_over_ridge * q + 1.;
   gamma = (m.total_gb == 0) ? 0. : gamma;
-  gamma = (m.num_gflops < 1e-9) ? 1. : gamma;
-  const bool bad_gamma = r.metrics && !(gamma >= 0 && gamma <= 1);
+  // A record without metrics takes the no-metrics strategy
+  // (resimplified.py:25-40): unchanged when small, else t * bw_ratio.  With
+  // gamma = 1 the roofline expressions below reduce to exactly that.
+  gamma = (m.num_gflops < 1e-9 || !r.metrics) ? 1. : gamma;
+  const bool bad_gamma = !(gamma >= 0 && gamma <= 1);
 
   // `a // wave_o == 0 and a // wave_d == 0`: the second test, and its division
   // by zero, happen only when the first holds (roofline.py:29-30).
@@ -186,15 +190,11 @@ __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn
   // roofline.py:32-45: (clk_ratio * dest_max_occ / origin_max_occ)^(1-gamma), both
   // counts in 1..32; roofline.py:48-64: bw^gamma * clk^(1-gamma) * sm^(1-gamma)
   const double gamma_compl = 1.0 - gamma;
-  const double log2_small =
-      p.log2_clk + log2_count<PERMUTE>(log2_lane, dest_max_occ) -
-      log2_count<PERMUTE>(log2_lane, m.origin_max_occ);
+  const double log2_small = p.log2_clk + log2_count<PERMUTE>(log2_lane, dest_max_occ) -
+                            log2_count<PERMUTE>(log2_lane, m.origin_max_occ);
   const double exponent =
       small ? gamma_compl * log2_small : gamma * p.log2_bw + gamma_compl * p.log2_clk_sm;
-  const double t_roofline = r.t * exp2_poly(exponent);
-  // resimplified.py:25-40
-  const double t_plain = small ? r.t : r.t * p.bw_ratio;
-  const double t = r.metrics ? t_roofline : t_plain;
+  const double t = r.t * exp2_poly(exponent);
   o.t = (status == HBT_ST_OK) ? t : __builtin_nan("");
   return o;
 }
