@@ -16,7 +16,9 @@ Two evaluations of the same weights:
 The arithmetic inside nn.Linear belongs to PyTorch (the reference pins
 torch==1.4.0, docker/Dockerfile:14; its source is not in the reference tree and
 the reference holds no vectors for it), so the only thing the reference itself
-fixes is the formula y = x W^T + b.  pins (tests/test_oracle_mlp.py): a
+fixes is the formula y = x W^T + b: beyond that formula this function is
+"parity unpinned" by the reference, and pinned by mathematics instead.
+pins (tests/test_oracle_mlp.py): a
 hand-computed 2-layer width-4 network; the all-ReLU-dead case (output =
 fc2.bias); linearity with ReLU inactive; agreement of the two evaluations;
 committed golden rows for the seed-0 networks (tests/golden/mlp_seed0.json).
