@@ -178,12 +178,14 @@ int hbt_wave_scale(const hbt_device_spec* origin, const hbt_device_spec* dests, 
     const int32_t nd = (n_dest - d0 < kMaxDestPerLaunch) ? (n_dest - d0) : kMaxDestPerLaunch;
     a.n_dest = nd;
     a.write_origin = (d0 == 0) ? 1 : 0;
-    const int64_t off = (int64_t)d0 * n;
-    a.out_time_ns = out_time_ns + off;
-    a.out_occ_dest = out_occ_dest ? out_occ_dest + off : nullptr;
-    a.out_wave_dest = out_wave_dest ? out_wave_dest + off : nullptr;
-    a.out_status = out_status ? out_status + off : nullptr;
-    for (int32_t k = 0; k < nd; ++k) a.dest[k] = make_dest_args(*origin, dests[d0 + k]);
+    for (int32_t k = 0; k < nd; ++k) {
+      const int64_t off = (int64_t)(d0 + k) * n;
+      a.dest[k] = make_dest_args(*origin, dests[d0 + k]);
+      a.out[k].time_ns = out_time_ns + off;
+      a.out[k].occ = out_occ_dest ? out_occ_dest + off : nullptr;
+      a.out[k].wave = out_wave_dest ? out_wave_dest + off : nullptr;
+      a.out[k].status = out_status ? out_status + off : nullptr;
+    }
     if (launch_wave_scale(a, vec, stream) != hipSuccess) return HBT_EHIP;
   }
   return HBT_OK;

@@ -33,6 +33,16 @@ struct OriginArgs {
   float inv_sms;       // 1 / origin.num_sms rounded to float
 };
 
+// Where one destination's results go (row d of the [n_dest][n] outputs).  Kept
+// per destination so that the kernel fetches these pointers when it reaches that
+// destination's stores rather than holding them from its first instruction.
+struct DestOut {
+  double* time_ns;
+  int32_t* occ;     // nullable
+  int32_t* wave;    // nullable
+  uint8_t* status;  // nullable
+};
+
 struct WaveScaleArgs {
   int64_t n;
   int32_t n_dest;
@@ -48,14 +58,11 @@ struct WaveScaleArgs {
   const double* dram_read_bytes;
   const double* dram_write_bytes;
   const uint8_t* has_metrics;  // nullable
-  double* out_time_ns;         // [n_dest][n]
   int32_t* out_occ_origin;     // [n], nullable
-  int32_t* out_occ_dest;       // [n_dest][n], nullable
   int32_t* out_wave_origin;    // [n], nullable
-  int32_t* out_wave_dest;      // [n_dest][n], nullable
-  uint8_t* out_status;         // [n_dest][n], nullable
   OriginArgs origin;
   DestArgs dest[kMaxDestPerLaunch];
+  DestOut out[kMaxDestPerLaunch];
 };
 
 OriginArgs make_origin_args(const hbt_device_spec& origin);

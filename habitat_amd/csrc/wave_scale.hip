@@ -108,7 +108,6 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
 
   for (int d = 0; d < a.n_dest; ++d) {
     const DestArgs& p = a.dest[d];
-    const int64_t row = (int64_t)d * a.n;  // uniform: goes into the base pointer
     double ot[R];
     int32_t occ_d[R], wave_d[R];
     uint8_t st[R];
@@ -117,10 +116,11 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
       const RecordOut o = dest_part<FAST, PERMUTE>(p, rin[k], mid[k], log2_lane);
       ot[k] = o.t; occ_d[k] = o.occ_d; wave_d[k] = o.wave_d; st[k] = o.status;
     }
-    store_r<double, R>(a.out_time_ns + row, i, ot);
-    if (a.out_occ_dest != nullptr) store_r<int32_t, R>(a.out_occ_dest + row, i, occ_d);
-    if (a.out_wave_dest != nullptr) store_r<int32_t, R>(a.out_wave_dest + row, i, wave_d);
-    if (a.out_status != nullptr) store_r<uint8_t, R>(a.out_status + row, i, st);
+    const DestOut& w = a.out[d];
+    store_r<double, R>(w.time_ns, i, ot);
+    if (w.occ != nullptr) store_r<int32_t, R>(w.occ, i, occ_d);
+    if (w.wave != nullptr) store_r<int32_t, R>(w.wave, i, wave_d);
+    if (w.status != nullptr) store_r<uint8_t, R>(w.status, i, st);
   }
 }
 
