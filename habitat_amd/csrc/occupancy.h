@@ -215,18 +215,22 @@ HBT_HD int32_t occupancy_fast(const OccDevice& d, int32_t block, const SmemAlloc
 
   // registers: 256 per-warp granularity, allocated per sub-partition; a block
   // must fit the per-block limit with its warps rounded up to the sub-partitions
-  const int32_t per_warp = ((mul_small(regs, ws) + 255) >> 8) << 8;
+  // (in units of 256 registers the per-warp allocation is at most 2^10 and the
+  // rounded warp count below 2^21: their product fits 32 bits, and comparing it
+  // with floor(regs_per_block / 256) is the comparison of the full sizes)
+  const int32_t per_warp256 = (mul_small(regs, ws) + 255) >> 8;
+  const int32_t per_warp = per_warp256 << 8;
   const int32_t sub_mask = (1 << d.sub_shift) - 1;
-  const uint32_t warps_up = (uint32_t)((warps + sub_mask) & ~sub_mask);
-  bool fits = (uint64_t)(uint32_t)per_warp * warps_up <= (uint64_t)(uint32_t)d.regs_per_block;
+  const int32_t warps_up = (warps + sub_mask) & ~sub_mask;
+  const int32_t block_regs256 = d.regs_per_block >> 8;
+  bool fits = mul_small(per_warp256, warps_up) <= block_regs256;
   const int32_t per_warp1 = per_warp > 0 ? per_warp : 1;
   const float rcp_per_warp = fast_rcp(per_warp1);
   const int32_t reg_warps = fast_div_r(d.regs_per_subpart, per_warp1, rcp_per_warp) << d.sub_shift;
   if (d.flags & kGp100) {
     // cc 6.0 must also fit a 4-sub-partition Pascal SM
-    const uint32_t warps_up4 = (uint32_t)((warps + 3) & ~3);
-    fits = fits &&
-           (uint64_t)(uint32_t)per_warp * warps_up4 <= (uint64_t)(uint32_t)d.regs_per_block &&
+    const int32_t warps_up4 = (warps + 3) & ~3;
+    fits = fits && mul_small(per_warp256, warps_up4) <= block_regs256 &&
            (per_warp == 0 ||
             (fast_div_r(d.regs_per_subpart4, per_warp1, rcp_per_warp) << 2) >= warps);
   }

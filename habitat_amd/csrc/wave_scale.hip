@@ -8,11 +8,13 @@
 // and the scaled time.
 //
 // Data layout: structure of arrays, one column per record field.  A thread owns
-// four consecutive records, so every int32 column is one 16-byte load per lane
-// (1 KiB per wavefront) and every fp64 column two; stores likewise.  Device
-// constants travel in the kernel-argument segment and live in SGPRs.  The
-// algorithmic traffic is 52 B read + 16 B written per record (5 x i32 + 4 x f64
-// in; f64 time + 2 x i32 occupancy out); optional columns add to that.
+// two consecutive records, so every int32 column is one 8-byte load per lane
+// and every fp64 column one 16-byte load; stores likewise.  All loads of a
+// thread are issued before any arithmetic and all stores after it, so that no
+// wait for a load also waits for a store.  Device constants travel in the
+// kernel-argument segment and live in SGPRs.  The algorithmic traffic is 52 B
+// read + 16 B written per record (5 x i32 + 4 x f64 in; f64 time + 2 x i32
+// occupancy out); optional columns add to that.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -33,7 +35,7 @@ namespace {
 using namespace dev;
 
 constexpr int kRecPerThread = 2;
-constexpr int kBlock = 256;
+constexpr int kBlock = 512;
 
 template <class T, int N>
 struct alignas(sizeof(T) * N) Pack { T v[N]; };
@@ -61,11 +63,13 @@ __device__ __forceinline__ void store_r(T* __restrict__ p, Index i, const T (&in
 }
 
 // Records i .. i+R-1 (all below n) for every destination of the launch.
-template <int R, bool FAST, bool PERMUTE, class Index>
+// SINGLE: the launch has one destination; its constants then sit at fixed
+// offsets of the argument segment and are fetched once, up front, instead of
+// inside a loop over destinations.
+template <int R, bool FAST, bool PERMUTE, bool SINGLE, class Index>
 __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
   const double log2_lane = PERMUTE ? kLog2Int[threadIdx.x & 63] : 0.0;
   int32_t nb[R], block[R], dyn[R], stat[R], regs[R], dregs[R];
-  uint8_t hm[R];
   double t[R], eff[R], rd[R], wr[R];
   load_r<int32_t, R>(a.num_blocks, i, nb);
   load_r<int32_t, R>(a.block_size, i, block);
@@ -82,11 +86,15 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
 #pragma unroll
     for (int k = 0; k < R; ++k) dregs[k] = -1;
   }
+  // The metrics flags stay packed in one register until the destination part
+  // needs them (see below), so that nothing waits for this load, the last one
+  // issued, before the arithmetic on the other columns starts.
+  uint32_t hm_bits = 0x01010101u;
   if (a.has_metrics != nullptr) {
-    load_r<uint8_t, R>(a.has_metrics, i, hm);
-  } else {
+    const Pack<uint8_t, R> v = *reinterpret_cast<const Pack<uint8_t, R>*>(a.has_metrics + (size_t)i);
+    hm_bits = 0;
 #pragma unroll
-    for (int k = 0; k < R; ++k) hm[k] = 1;
+    for (int k = 0; k < R; ++k) hm_bits |= (uint32_t)v.v[k] << (8 * k);
   }
 
   RecordIn rin[R];
@@ -94,19 +102,17 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
 #pragma unroll
   for (int k = 0; k < R; ++k) {
     rin[k] = RecordIn{nb[k], block[k], smem_sum(stat[k], dyn[k]), regs[k], dregs[k],
-                      hm[k] != 0, t[k], eff[k], rd[k], wr[k]};
+                      true, t[k], eff[k], rd[k], wr[k]};
     mid[k] = origin_part<FAST>(a.origin, rin[k]);
   }
-
-  if (a.write_origin) {
-    int32_t occ_o[R], wave_o[R];
+  // Opaque to the optimiser: keeps the unpacking of the flags from moving up
+  // to the load.
+  asm volatile("" : "+v"(hm_bits));
 #pragma unroll
-    for (int k = 0; k < R; ++k) { occ_o[k] = mid[k].occ_o; wave_o[k] = mid[k].wave_o; }
-    if (a.out_occ_origin != nullptr) store_r<int32_t, R>(a.out_occ_origin, i, occ_o);
-    if (a.out_wave_origin != nullptr) store_r<int32_t, R>(a.out_wave_origin, i, wave_o);
-  }
+  for (int k = 0; k < R; ++k) rin[k].metrics = ((hm_bits >> (8 * k)) & 0xffu) != 0;
 
-  for (int d = 0; d < a.n_dest; ++d) {
+  const int n_dest = SINGLE ? 1 : a.n_dest;
+  for (int d = 0; d < n_dest; ++d) {
     const DestArgs& p = a.dest[d];
     double ot[R];
     int32_t occ_d[R], wave_d[R];
@@ -122,9 +128,20 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
     if (w.wave != nullptr) store_r<int32_t, R>(w.wave, i, wave_d);
     if (w.status != nullptr) store_r<uint8_t, R>(w.status, i, st);
   }
+
+  // Origin columns last: a store issued between the loads and the arithmetic
+  // that consumes them would have to be waited for together with the loads
+  // (one counter tracks both).
+  if (a.write_origin) {
+    int32_t occ_o[R], wave_o[R];
+#pragma unroll
+    for (int k = 0; k < R; ++k) { occ_o[k] = mid[k].occ_o; wave_o[k] = mid[k].wave_o; }
+    if (a.out_occ_origin != nullptr) store_r<int32_t, R>(a.out_occ_origin, i, occ_o);
+    if (a.out_wave_origin != nullptr) store_r<int32_t, R>(a.out_wave_origin, i, wave_o);
+  }
 }
 
-template <int R, bool FAST, class Index>
+template <int R, bool FAST, bool SINGLE, class Index>
 __global__ __launch_bounds__(kBlock) void wave_scale_kernel(const WaveScaleArgs a) {
   const Index thread = (Index)blockIdx.x * kBlock + threadIdx.x;
   const Index i = thread * R;
@@ -134,10 +151,10 @@ __global__ __launch_bounds__(kBlock) void wave_scale_kernel(const WaveScaleArgs 
   // record at a time.
   const Index wave_end = ((thread | 63) + 1) * R;
   if (wave_end <= n) {
-    process<R, FAST, true, Index>(a, i);
+    process<R, FAST, true, SINGLE, Index>(a, i);
   } else {
     const Index end = (i + R < n) ? i + R : n;
-    for (Index j = i; j < end; ++j) process<1, FAST, false, Index>(a, j);
+    for (Index j = i; j < end; ++j) process<1, FAST, false, SINGLE, Index>(a, j);
   }
 }
 
@@ -145,8 +162,12 @@ template <int R, bool FAST, class Index>
 void launch(const WaveScaleArgs& args, hipStream_t stream) {
   const int64_t threads = (args.n + R - 1) / R;
   const int64_t blocks = (threads + kBlock - 1) / kBlock;
-  hipLaunchKernelGGL((wave_scale_kernel<R, FAST, Index>), dim3((unsigned)blocks), dim3(kBlock), 0,
-                     stream, args);
+  if (args.n_dest == 1)
+    hipLaunchKernelGGL((wave_scale_kernel<R, FAST, true, Index>), dim3((unsigned)blocks),
+                       dim3(kBlock), 0, stream, args);
+  else
+    hipLaunchKernelGGL((wave_scale_kernel<R, FAST, false, Index>), dim3((unsigned)blocks),
+                       dim3(kBlock), 0, stream, args);
 }
 
 template <int R, bool FAST>

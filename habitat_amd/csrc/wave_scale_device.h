@@ -126,9 +126,12 @@ __device__ __forceinline__ RecordMid origin_part(const OriginArgs& o, const Reco
   m.small_o = r.nb >= 0 && r.nb < m.wave_o;
   m.origin_max_occ =
       ceil_div_small<FAST>(m.small_o ? r.nb : 0, o.dev.num_sms, o.inv_sms);
-  // roofline.py:72-76, same operation order (the three divisions by 1024 are
-  // exact scalings)
-  m.total_gb = (r.rd + r.wr) / 1024 / 1024 / 1024;
+  // roofline.py:72-76, same operation order.  The three divisions by 1024 are
+  // exact scalings, done here as one by 2^-30.  (Below 2^-992 bytes, where a
+  // quotient is subnormal and one rounding is not three, the last bits of
+  // total_gb reach no output: gamma is then forced to 1 by num_gflops < 1e-9
+  // or lies within 1e-290 of 0.)
+  m.total_gb = (r.rd + r.wr) * 0x1p-30;
   const double gflops_per_second = div_const<C100>(r.eff) * o.peak_gflops;
   m.num_gflops = div_const<C1e9>(gflops_per_second * r.t);
   return m;
