@@ -15,6 +15,9 @@ inputs resident in HBM.  Prints ONE JSON line:
   large         the same kernel at 64 M records (beyond the 256 MB last-level cache)
   mlp           the fused MFMA MLP (configs[2], conv2d, 1 M rows): rows/s, its
                 roofline against fp32 MFMA peak and a torch-CPU fp32 baseline
+  sweep         configs[4]: one ResNet-50-shaped trace predicted for 256 devices
+                (fused per-pass sums + MLP rows + ratio kernel), eager and as a
+                replayed HIP graph, next to the per-device CPU path
 Only one GPU is used; --gpus above 1 exits.
 """
 import argparse
@@ -51,6 +54,9 @@ def parse():
     ap.add_argument("--no-mlp", action="store_true")
     ap.add_argument("--no-large", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true",
+                    help="skip configs[4] (one ResNet-50-shaped trace against 256 devices)")
+    ap.add_argument("--sweep-devices", type=int, default=256)
     ap.add_argument("--no-ceilings", action="store_true",
                     help="skip measuring the box's own copy bandwidth and FMA/MFMA rates")
     ap.add_argument("--mlp-other-kinds", default="linear,bmm,lstm",
@@ -111,6 +117,121 @@ def tile_records(rec, n):
     base = rec["num_blocks"].shape[0]
     reps = (n + base - 1) // base
     return {k: np.tile(v, reps)[:n] for k, v in rec.items()}
+
+
+def sweep_bench(args, origin):
+    """configs[4]: predicted iteration time of one trace on D devices."""
+    import numpy as np
+    import torch
+    from habitat_amd import synthetic
+    from habitat_amd.analysis import predictor as P
+    from habitat_amd.analysis.mlp.mlp import RuntimePredictor
+    from habitat_amd.analysis.predictor import Predictor
+    D = args.sweep_devices
+    trace = synthetic.resnet50_trace(origin, batch=32, seed=3)
+    preds = {}
+    for kind in ("conv2d", "linear"):
+        torch.manual_seed(0)
+        rp = RuntimePredictor(kind, 8, 1024)
+        _, mu, sigma = synthetic.mlp_features(kind, 2048, seed=2)
+        rp.set_normalization(mu, sigma)
+        preds[kind] = rp
+    predictor = Predictor(mlp_predictors=preds)
+    devices, feats = synthetic.device_sweep(D, seed=1)
+    device_features = {d.name: list(f) for d, f in zip(devices, feats)}
+    device_features[origin.name] = [16, 900, 80, 14.028]
+
+    t0 = time.perf_counter()
+    plan = predictor.plan_trace(trace)
+    call = plan.prepare(devices, device_features)
+    torch.cuda.synchronize()
+    prepare_ms = (time.perf_counter() - t0) * 1e3
+    eager_wall, eager_gpu = time_steps(call.launch, 50, 5)
+    totals = call.launch().total_ms
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call.launch()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = call.launch()
+    graph_wall, graph_gpu = time_steps(graph.replay, 50, 5)
+    torch.cuda.synchronize()
+    same = bool(torch.allclose(captured.total_ms, totals, rtol=1e-12, atol=0))
+    n_kernels = len(plan.kernels)
+    n_special = sum(len(v[0]) for v in plan.special.values())
+    out = {"workload": "configs[4]: ResNet-50-shaped trace (%d operations, %d kernel records in "
+                       "%d passes, %d MLP-predicted operations), V100 origin, %d synthetic devices"
+                       % (len(trace.operations), n_kernels, len(plan.pass_owner), n_special, D),
+           "devices": D, "prepare_ms_once": prepare_ms,
+           "eager": {"ms_per_sweep": eager_wall, "gpu_ms_per_sweep": eager_gpu,
+                     "device_predictions_per_s": D / (eager_wall * 1e-3)},
+           "hip_graph": {"ms_per_sweep": graph_wall, "gpu_ms_per_sweep": graph_gpu,
+                         "device_predictions_per_s": D / (graph_wall * 1e-3),
+                         "replay_equals_eager": same},
+           "unit": "predicted (trace, device) pairs per second"}
+    if not args.no_cpu:
+        # the reference's shape of work on the host: per device, one Python call
+        # chain per kernel and two batch-1 MLP forwards per special operation
+        from habitat_amd.analysis.metrics import Metric
+        from oracle import lib as olib
+        from oracle import mlp as omlp
+        from oracle import predictor as opred
+        from oracle import wave_scaling as ows
+        o = olib.make_device(**origin.as_dict())
+        metrics = (Metric.SinglePrecisionFLOPEfficiency, Metric.DRAMReadBytes,
+                   Metric.DRAMWriteBytes)
+        sample = devices[:2]
+        t0 = time.perf_counter()
+        cpu_totals = []
+        for dev in sample:
+            d = olib.make_device(**dev.as_dict())
+            total = 0.0
+            for op in trace.operations:
+                if op.name in preds:
+                    rp = preds[op.name]
+                    a = P._ARGUMENTS[op.name](op)
+                    f = [a[x] for x in rp.model.features]
+                    sd = rp.model.state_dict()
+                    y_d = omlp.forward_fp32(sd, np.array([f + device_features[dev.name]]),
+                                            rp.mu, rp.sigma)[0]
+                    y_o = omlp.forward_fp32(sd, np.array([f + device_features[origin.name]]),
+                                            rp.mu, rp.sigma)[0]
+                    total += opred.special_op_ms(op.run_time_ms, float(y_d), float(y_o))
+                    continue
+                for rt in (op.forward, op.backward):
+                    if rt is None:
+                        continue
+                    pk = []
+                    for k in rt.kernels:
+                        try:
+                            m = tuple(k.get_metric(x) for x in metrics)
+                        except AttributeError:
+                            m = None
+                        nb, block, dyn, stat, regs, t_ns = P.kernel_fields(k)
+                        row = {"num_blocks": nb, "block_size": block, "dynamic_smem": dyn,
+                               "static_smem": stat, "regs_per_thread": regs, "run_time_ns": t_ns,
+                               "flop_sp_efficiency": m[0] if m else 0.0,
+                               "dram_read_bytes": m[1] if m else 0.0,
+                               "dram_write_bytes": m[2] if m else 0.0}
+                        pk.append(ows.unified(row, o, d, has_metrics=m is not None))
+                    total += opred.wave_scaled_pass_ms(rt.run_time_ms,
+                                                       [k.run_time_ns for k in rt.kernels], pk)
+            cpu_totals.append(total)
+        dt = time.perf_counter() - t0
+        got = totals[:len(sample)].cpu().numpy()
+        out["cpu_baseline"] = {
+            "value": len(sample) / dt, "unit": "predicted (trace, device) pairs per second",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "oracle (Python call chain per kernel, two batch-1 torch-CPU fp32 MLP "
+                      "forwards per MLP-predicted operation, as the reference does) for the "
+                      "first %d devices" % len(sample),
+            "max_rel_diff_vs_gpu": float(np.max(np.abs(got - np.array(cpu_totals)) /
+                                                np.abs(np.array(cpu_totals))))}
+    return out
 
 
 def main():
@@ -269,6 +390,10 @@ def main():
         if others:
             mlp["other_kinds"] = others
         result["mlp"] = mlp
+
+    # ---------------- configs[4]: one trace, a sweep of destination devices ----------------
+    if not args.no_sweep:
+        result["sweep"] = sweep_bench(args, origin)
 
     # ---------------- what this box itself can do (ceilings under the published peaks) ----------
     if not args.no_ceilings:

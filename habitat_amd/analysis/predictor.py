@@ -316,3 +316,12 @@ class Predictor:
         (a habitat_amd.analysis.sweep.TraceSweep)."""
         from habitat_amd.analysis.sweep import predict_trace_sweep
         return predict_trace_sweep(self, trace, dest_devices, device_features)
+
+    def plan_trace(self, trace):
+        """The destination-independent part of a sweep, resident on the GPU (a
+        habitat_amd.analysis.sweep.TracePlan): build it once per trace, then
+        `plan.run(dest_devices)` per set of destinations, or
+        `plan.prepare(dest_devices).launch()` to repeat or graph-capture the
+        GPU work."""
+        from habitat_amd.analysis.sweep import TracePlan
+        return TracePlan(self, trace)

@@ -37,83 +37,163 @@ class TraceSweep:
         self.bad_records = None     # int32 [D]: records on which the reference would raise
 
 
-def predict_trace_sweep(predictor, trace, dest_devices, device_features=None):
-    from habitat_amd.analysis import predictor as P
-    dests = list(dest_devices)
-    D = len(dests)
-    origin = trace.device
-    mode = P._BUILTIN.get(predictor._wave_scaling_strategy)
-    if mode is None:
-        raise ValueError("device sweeps need one of the built-in wave-scaling strategies")
+class TracePlan:
+    """What a sweep needs of one trace, independent of the destinations and
+    resident on the GPU: the kernel records of every wave-scaled pass with their
+    pass numbers, the pass overheads, and per MLP kind the operation features
+    and measured times.  Build once per trace, then `run` (or `prepare` +
+    `launch`) per set of destinations."""
 
-    def feats_of(dev):
-        if device_features is not None and dev.name in device_features:
-            return list(device_features[dev.name])
-        return get_device_features(dev.name, ["mem", "mem_bw", "num_sm", "single"])
+    def __init__(self, predictor, trace):
+        from habitat_amd.analysis import predictor as P
+        self.predictor = predictor
+        self.origin = trace.device
+        self.mode = P._BUILTIN.get(predictor._wave_scaling_strategy)
+        if self.mode is None:
+            raise ValueError("device sweeps need one of the built-in wave-scaling strategies")
+        self.gpu = torch.device("cuda", torch.cuda.current_device())
+        kernels, segment, overheads, owners = [], [], [], []
+        const_ms = 0.0
+        special = {}
+        for idx, op in enumerate(trace.operations):
+            if op.name not in SPECIAL_OPERATIONS:
+                for which, rt in (("forward", op.forward), ("backward", op.backward)):
+                    if rt is None:
+                        continue
+                    overhead = ms_to_ns(rt.run_time_ms) - sum(k.run_time_ns for k in rt.kernels)
+                    overhead = 0 if overhead < 0 else overhead
+                    const_ms += overhead / 1e6
+                    segment.extend([len(owners)] * len(rt.kernels))
+                    kernels.extend(rt.kernels)
+                    overheads.append(overhead)
+                    owners.append((idx, which))
+            elif op.name in P._ARGUMENTS:
+                special.setdefault(op.name, []).append(idx)
+            else:
+                const_ms += op.run_time_ms
+        self.const_ms = const_ms
+        self.kernels = kernels
+        self.pass_overhead_ns = np.asarray(overheads, np.float64)
+        self.pass_owner = owners
+        self.n_seg = max(len(owners), 1)
+        self.segment = (torch.tensor(segment, dtype=torch.int32, device=self.gpu)
+                        if kernels else None)
+        self._records = {}
+        self.special = {}
+        for kind, idxs in special.items():
+            pred = predictor._mlp(kind)
+            ops = [trace.operations[i] for i in idxs]
+            feats = []
+            for op in ops:
+                a = P._ARGUMENTS[kind](op)
+                feats.append([a[x] for x in pred.model.features])
+            self.special[kind] = (
+                idxs, pred,
+                torch.tensor(np.asarray(feats, np.float64), device=self.gpu),          # [O, F]
+                torch.tensor([op.run_time_ms for op in ops], dtype=torch.float64, device=self.gpu))
 
-    res = TraceSweep()
-    kernels, segment, overheads, owners = [], [], [], []
-    const_ms = 0.0
-    special = {}
-    for idx, op in enumerate(trace.operations):
-        if op.name not in SPECIAL_OPERATIONS:
-            for which, rt in (("forward", op.forward), ("backward", op.backward)):
-                if rt is None:
-                    continue
-                overhead = ms_to_ns(rt.run_time_ms) - sum(k.run_time_ns for k in rt.kernels)
-                overhead = 0 if overhead < 0 else overhead
-                const_ms += overhead / 1e6
-                segment.extend([len(owners)] * len(rt.kernels))
-                kernels.extend(rt.kernels)
-                overheads.append(overhead)
-                owners.append((idx, which))
-        elif op.name in P._ARGUMENTS:
-            special.setdefault(op.name, []).append(idx)
+    def _records_for(self, dest):
+        """Kernel records with the register column resolved for `dest`'s
+        architecture (the look-up depends on nothing else of the destination)."""
+        from habitat_amd.analysis import predictor as P
+        from habitat_amd.analysis.wave_scaling.metadata import NullMetadataManager
+        meta = self.predictor._kernel_metadata
+        key = None if isinstance(meta, NullMetadataManager) else dest.compute_capability
+        if key not in self._records:
+            self._records[key] = P.records_from_kernels(self.kernels, dest, meta, self.mode)
+        return self._records[key]
+
+    def prepare(self, dest_devices, device_features=None):
+        """Everything that allocates or copies for one set of destinations: the
+        device-resident destination tables and the MLP device-feature rows.
+        Returns a SweepCall whose `launch()` only enqueues kernels."""
+        return SweepCall(self, list(dest_devices), device_features)
+
+    def run(self, dest_devices, device_features=None):
+        return self.prepare(dest_devices, device_features).launch()
+
+
+class SweepCall:
+    """A prepared sweep: `launch()` enqueues its kernels on the current stream
+    and returns a TraceSweep of GPU tensors, without synchronising and without
+    reading anything back, so it can be repeated or captured in a HIP graph."""
+
+    def __init__(self, plan, dests, device_features):
+        self.plan = plan
+        self.dests = dests
+
+        def feats_of(dev):
+            if device_features is not None and dev.name in device_features:
+                return list(device_features[dev.name])
+            return get_device_features(dev.name, ["mem", "mem_bw", "num_sm", "single"])
+
+        self.groups = []
+        if plan.kernels:
+            by_arch = {}
+            for i, d in enumerate(dests):
+                by_arch.setdefault(d.compute_capability, []).append(i)
+            whole = len(by_arch) == 1
+            for idxs in by_arch.values():
+                rec = plan._records_for(dests[idxs[0]])
+                table = DeviceTable(plan.origin, [dests[i] for i in idxs])
+                at = None if whole else torch.tensor(idxs, device=plan.gpu)
+                self.groups.append((rec, table, at))
+        self.dev_feats = None
+        self.streams = [torch.cuda.Stream(plan.gpu) for _ in plan.special]   # default priority
+        if plan.special:
+            self.dev_feats = torch.tensor(
+                np.asarray([feats_of(d) for d in dests] + [feats_of(plan.origin)], np.float64),
+                device=plan.gpu)                                                      # [D + 1, 4]
+
+    def launch(self):
+        plan, D = self.plan, len(self.dests)
+        res = TraceSweep()
+        res.pass_overhead_ns = plan.pass_overhead_ns
+        res.pass_owner = plan.pass_owner
+        total = torch.full((D,), plan.const_ms, dtype=torch.float64, device=plan.gpu)
+        if self.groups:
+            if len(self.groups) == 1 and self.groups[0][2] is None:
+                rec, table, _ = self.groups[0]
+                res.pass_kernel_ns, res.bad_records = wave_scale_sum(rec, table, plan.segment,
+                                                                     plan.n_seg)
+            else:
+                res.pass_kernel_ns = torch.zeros((D, plan.n_seg), dtype=torch.float64,
+                                                 device=plan.gpu)
+                res.bad_records = torch.zeros((D,), dtype=torch.int32, device=plan.gpu)
+                for rec, table, at in self.groups:
+                    sums, bad = wave_scale_sum(rec, table, plan.segment, plan.n_seg)
+                    res.pass_kernel_ns[at] = sums
+                    res.bad_records[at] = bad
+            total += res.pass_kernel_ns.sum(dim=1) / 1e6
+            total = torch.where(res.bad_records > 0, torch.full_like(total, float("nan")), total)
         else:
-            const_ms += op.run_time_ms
-    res.pass_overhead_ns = np.asarray(overheads, np.float64)
-    res.pass_owner = owners
+            res.pass_kernel_ns = torch.zeros((D, plan.n_seg), dtype=torch.float64, device=plan.gpu)
+            res.bad_records = torch.zeros((D,), dtype=torch.int32, device=plan.gpu)
+        # One MLP launch per kind, each on a stream of its own: a kind with few
+        # operations fills a fraction of the GPU, so the kinds run side by side.
+        main = torch.cuda.current_stream(plan.gpu)
+        preds = {}
+        for (kind, (idxs, pred, op_feats, ms)), side in zip(plan.special.items(), self.streams):
+            O = op_feats.shape[0]
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                rows = torch.cat([op_feats.unsqueeze(0).expand(D + 1, O, -1),
+                                  self.dev_feats.unsqueeze(1).expand(D + 1, O, 4)], dim=2)
+                y = pred.predict_batch(rows.reshape((D + 1) * O, -1)).view(D + 1, O)
+            rows.record_stream(main)
+            y.record_stream(main)
+            preds[kind] = y
+        for side in self.streams:
+            main.wait_stream(side)
+        for kind, (idxs, pred, op_feats, ms) in plan.special.items():
+            res.special_ms[kind] = ratio_scale(preds[kind], ms, D, totals=total)
+            res.special_owner[kind] = idxs
+        res.total_ms = total
+        return res
 
-    gpu = torch.device("cuda", torch.cuda.current_device())
-    total = torch.full((D,), const_ms, dtype=torch.float64, device=gpu)
-    res.bad_records = torch.zeros((D,), dtype=torch.int32, device=gpu)
-    n_seg = max(len(owners), 1)
-    res.pass_kernel_ns = torch.zeros((D, n_seg), dtype=torch.float64, device=gpu)
-    if kernels:
-        seg = torch.tensor(segment, dtype=torch.int32, device=gpu)
-        # The register look-up depends on the destination's architecture: one
-        # launch per group of destinations that share it (one group without a table).
-        groups = {}
-        for i, d in enumerate(dests):
-            groups.setdefault(d.compute_capability, []).append(i)
-        for idxs in groups.values():
-            rec = P.records_from_kernels(kernels, dests[idxs[0]], predictor._kernel_metadata, mode)
-            table = DeviceTable(origin, [dests[i] for i in idxs])
-            sums, bad = wave_scale_sum(rec, table, seg, n_seg)
-            at = torch.tensor(idxs, device=gpu)
-            res.pass_kernel_ns[at] = sums
-            res.bad_records[at] = bad
-        total += res.pass_kernel_ns.sum(dim=1) / 1e6
-        total = torch.where(res.bad_records > 0, torch.full_like(total, float("nan")), total)
 
-    for kind, idxs in special.items():
-        pred = predictor._mlp(kind)
-        ops = [trace.operations[i] for i in idxs]
-        op_feats = []
-        for op in ops:
-            a = P._ARGUMENTS[kind](op)
-            op_feats.append([a[x] for x in pred.model.features])
-        op_feats = np.asarray(op_feats, np.float64)                        # [O, F]
-        dev_feats = np.asarray([feats_of(d) for d in dests] + [feats_of(origin)], np.float64)
-        O = op_feats.shape[0]
-        rows = np.concatenate([np.repeat(op_feats[None], D + 1, axis=0),
-                               np.repeat(dev_feats[:, None], O, axis=1)], axis=2)
-        y = pred.predict_batch(rows.reshape((D + 1) * O, -1)).view(D + 1, O)
-        ms = torch.tensor([op.run_time_ms for op in ops], dtype=torch.float64, device=gpu)
-        res.special_ms[kind] = ratio_scale(y, ms, D, totals=total)
-        res.special_owner[kind] = idxs
-    res.total_ms = total
-    return res
+def predict_trace_sweep(predictor, trace, dest_devices, device_features=None):
+    return TracePlan(predictor, trace).run(dest_devices, device_features)
 
 
 def predict_trace_times(predictor, trace, dest_devices, device_features=None):

@@ -154,6 +154,70 @@ def test_end_to_end_256_device_sweep():
     assert np.corrcoef(rank(bw), rank(totals))[0, 1] < -0.3
 
 
+def _sweep_fixture(n_devices):
+    origin = Device.V100
+    trace = synthetic.resnet50_trace(origin, batch=32, seed=3)
+    preds = {}
+    for kind in ("conv2d", "linear"):
+        torch.manual_seed(0)
+        rp = RuntimePredictor(kind, 8, 1024)
+        x, mu, sigma = synthetic.mlp_features(kind, 2048, seed=2)
+        rp.set_normalization(mu, sigma)
+        preds[kind] = rp
+    predictor = Predictor(mlp_predictors=preds)
+    devices, feats = synthetic.device_sweep(n_devices, seed=1)
+    device_features = {d.name: list(f) for d, f in zip(devices, feats)}
+    device_features[origin.name] = [16, 900, 80, 14.028]
+    return predictor, trace, devices, device_features
+
+
+def test_plan_reuse_and_subsets_agree_with_one_shot_sweep():
+    predictor, trace, devices, feats = _sweep_fixture(24)
+    whole = predictor.predict_trace_sweep(trace, devices, feats).total_ms.cpu().numpy()
+    plan = predictor.plan_trace(trace)
+    again = plan.run(devices, feats).total_ms.cpu().numpy()
+    np.testing.assert_array_equal(whole, again)
+    part = plan.run(devices[5:9], feats).total_ms.cpu().numpy()
+    # a destination's total does not depend on which others share the launch;
+    # the MLP rows and the order of the fp64 atomic adds do, to rounding
+    np.testing.assert_allclose(part, whole[5:9], rtol=1e-12)
+
+
+def test_prepared_sweep_replays_in_a_hip_graph():
+    """The GPU work of a prepared sweep allocates through torch only and never
+    synchronises, so it can be captured once and replayed; every replay, with
+    eager work and synchronisations in between, gives the eager totals."""
+    predictor, trace, devices, feats = _sweep_fixture(32)
+    call = predictor.plan_trace(trace).prepare(devices, feats)
+    eager = call.launch()
+    torch.cuda.synchronize()
+    want_total = eager.total_ms.clone()
+    want_pass = eager.pass_kernel_ns.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):          # warm-up on the capture stream
+            call.launch()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = call.launch()
+    for replay in range(4):
+        captured.total_ms.fill_(-1.0)
+        captured.pass_kernel_ns.fill_(-1.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        # order of the fp64 atomic adds within a pass differs between launches
+        torch.testing.assert_close(captured.total_ms, want_total, rtol=1e-12, atol=0)
+        torch.testing.assert_close(captured.pass_kernel_ns, want_pass, rtol=1e-12, atol=0)
+        assert int(captured.bad_records.sum().item()) == 0
+        # the program's own eager work between replays
+        other = call.launch().total_ms
+        torch.cuda.synchronize()
+        torch.testing.assert_close(other, want_total, rtol=1e-12, atol=0)
+
+
 def test_device_table_argument_checks():
     with pytest.raises(ValueError):
         DeviceTable(Device.V100, [])
