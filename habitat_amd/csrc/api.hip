@@ -149,17 +149,20 @@ int hbt_wave_scale(const hbt_device_spec* origin, const hbt_device_spec* dests, 
                             out_occ_origin, out_occ_dest, out_wave_origin, out_wave_dest};
   const void* f64_cols[] = {run_time_ns, flop_sp_efficiency, dram_read_bytes, dram_write_bytes,
                             out_time_ns};
+  // The vectorised kernel accesses kVectorRecords elements at a time: every
+  // column, and every destination's row of an output ([n_dest][n]), must be
+  // aligned to that many elements.
   bool vec = true;
   for (const void* p : i32_cols) {
     if (!aligned(p, 4)) return HBT_EALIGN;
-    vec = vec && aligned(p, 16);
+    vec = vec && aligned(p, 4 * kVectorRecords);
   }
   for (const void* p : f64_cols) {
     if (!aligned(p, 8)) return HBT_EALIGN;
-    vec = vec && aligned(p, 32);
+    vec = vec && aligned(p, 8 * kVectorRecords);
   }
-  vec = vec && aligned(has_metrics, 4) && aligned(out_status, 4);
-  if (n_dest > 1 && (n % 4) != 0) vec = false;
+  vec = vec && aligned(has_metrics, kVectorRecords) && aligned(out_status, kVectorRecords);
+  if (n_dest > 1 && (n % kVectorRecords) != 0) vec = false;
 
   if (hbt_device_count() <= 0) return HBT_EHIP;
 

@@ -12,6 +12,10 @@ namespace hbt {
 // Destinations handled by one launch; more are processed in successive launches.
 constexpr int kMaxDestPerLaunch = 8;
 
+// Consecutive records one thread of the vectorised kernel owns: each of its
+// column accesses is one load or store of this many elements.
+constexpr int kVectorRecords = 2;
+
 // Everything about one (origin, destination) pair that does not depend on the
 // record, computed in fp64 on the host in the reference's operation order
 // (analyzer/habitat/analysis/wave_scaling/roofline.py:48-64, :107-108).
@@ -68,7 +72,8 @@ struct WaveScaleArgs {
 OriginArgs make_origin_args(const hbt_device_spec& origin);
 DestArgs make_dest_args(const hbt_device_spec& origin, const hbt_device_spec& dest);
 
-// `vectorised` needs every column 16-byte aligned (and n % 4 == 0 when n_dest > 1).
+// `vectorised` needs every column, and every destination's row of the outputs,
+// aligned to kVectorRecords elements of its type.
 hipError_t launch_wave_scale(const WaveScaleArgs& args, bool vectorised, hipStream_t stream);
 
 }  // namespace hbt

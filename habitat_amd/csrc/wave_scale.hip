@@ -34,7 +34,7 @@ namespace {
 
 using namespace dev;
 
-constexpr int kRecPerThread = 2;
+constexpr int kRecPerThread = kVectorRecords;
 constexpr int kBlock = 512;
 
 template <class T, int N>

@@ -154,7 +154,7 @@ def test_slow_division_path_with_huge_device_and_record_values():
         check(rec, origin, [dest], out)
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 255, 256, 257, 1023, 1025])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 130, 255, 256, 257, 258, 386, 1023, 1025, 2050])
 def test_ragged_sizes_single_and_multi_destination(n):
     rec, _ = synthetic.kernel_records(n, Device.V100, seed=n)
     dests = [Device.MI355X, Device.T4, Device.P100]
