@@ -150,7 +150,13 @@ struct RecordOut {
 // it from the table in memory.
 template <bool PERMUTE>
 __device__ __forceinline__ double log2_count(double log2_lane, int32_t count) {
-  if (PERMUTE) return __shfl(log2_lane, count & 63);
+  if (PERMUTE) {
+    // lane `count` of the wavefront (the hardware takes the lane number modulo 64)
+    const int addr = count << 2;
+    const int lo = __builtin_amdgcn_ds_bpermute(addr, __double2loint(log2_lane));
+    const int hi = __builtin_amdgcn_ds_bpermute(addr, __double2hiint(log2_lane));
+    return __hiloint2double(hi, lo);
+  }
   return kLog2Int[count & 63];
 }
 
