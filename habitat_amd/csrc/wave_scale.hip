@@ -37,29 +37,51 @@ using namespace dev;
 constexpr int kRecPerThread = kVectorRecords;
 constexpr int kBlock = 512;
 
+// N consecutive elements as one register group (a scalar when N is 1).
 template <class T, int N>
-struct alignas(sizeof(T) * N) Pack { T v[N]; };
+struct VecOf { using type = T __attribute__((ext_vector_type(N))); };
+template <class T>
+struct VecOf<T, 1> { using type = T; };
+
+template <class T, int N>
+__device__ __forceinline__ T vec_get(const typename VecOf<T, N>::type& v, int k) {
+  if constexpr (N == 1) return v;
+  else return v[k];
+}
+
+template <class T, int N>
+__device__ __forceinline__ void vec_set(typename VecOf<T, N>::type& v, int k, T x) {
+  if constexpr (N == 1) v = x;
+  else v[k] = x;
+}
 
 // R consecutive elements starting at element i, all in range: one vector
 // access.  Index is uint32_t when every byte offset of the launch fits 32 bits
 // (the address is then a uniform 64-bit base plus a 32-bit lane offset, which
 // costs no 64-bit vector arithmetic), else uint64_t.
+//
+// Every column is read once and every output written once, so both directions
+// carry the non-temporal hint: the lines are not kept in L2 or the last-level
+// cache at the expense of each other.  Measured against plain accesses:
+// 745 vs 825 us at 64 M records, 13.0 vs 13.8 us at 1 M.
 template <class T, int R, class Index>
 __device__ __forceinline__ void load_r(const T* __restrict__ p, Index i, T (&out)[R]) {
+  using V = typename VecOf<T, R>::type;
   const Index byte = i * (Index)sizeof(T);
-  const Pack<T, R> v =
-      *reinterpret_cast<const Pack<T, R>*>(reinterpret_cast<const char*>(p) + (size_t)byte);
+  const V v = __builtin_nontemporal_load(
+      reinterpret_cast<const V*>(reinterpret_cast<const char*>(p) + (size_t)byte));
 #pragma unroll
-  for (int k = 0; k < R; ++k) out[k] = v.v[k];
+  for (int k = 0; k < R; ++k) out[k] = vec_get<T, R>(v, k);
 }
 
 template <class T, int R, class Index>
 __device__ __forceinline__ void store_r(T* __restrict__ p, Index i, const T (&in)[R]) {
-  Pack<T, R> v;
+  using V = typename VecOf<T, R>::type;
+  V v;
 #pragma unroll
-  for (int k = 0; k < R; ++k) v.v[k] = in[k];
+  for (int k = 0; k < R; ++k) vec_set<T, R>(v, k, in[k]);
   const Index byte = i * (Index)sizeof(T);
-  *reinterpret_cast<Pack<T, R>*>(reinterpret_cast<char*>(p) + (size_t)byte) = v;
+  __builtin_nontemporal_store(v, reinterpret_cast<V*>(reinterpret_cast<char*>(p) + (size_t)byte));
 }
 
 // Records i .. i+R-1 (all below n) for every destination of the launch.
@@ -91,10 +113,11 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
   // issued, before the arithmetic on the other columns starts.
   uint32_t hm_bits = 0x01010101u;
   if (a.has_metrics != nullptr) {
-    const Pack<uint8_t, R> v = *reinterpret_cast<const Pack<uint8_t, R>*>(a.has_metrics + (size_t)i);
+    uint8_t v[R];
+    load_r<uint8_t, R>(a.has_metrics, i, v);
     hm_bits = 0;
 #pragma unroll
-    for (int k = 0; k < R; ++k) hm_bits |= (uint32_t)v.v[k] << (8 * k);
+    for (int k = 0; k < R; ++k) hm_bits |= (uint32_t)v[k] << (8 * k);
   }
 
   RecordIn rin[R];
