@@ -22,6 +22,7 @@ from habitat_amd.analysis.mlp.mlp import RuntimePredictor
 from habitat_amd.analysis.operation import PredictedOperation
 from habitat_amd.analysis.run_time import (RunTimePrediction, RunTimePurePrediction, ms_to_ns)
 from habitat_amd.analysis.wave_scaling.batch import KernelRecords, wave_scale
+from habitat_amd.analysis.wave_scaling.cdna import cdna_wave_scaling, native_description
 from habitat_amd.analysis.wave_scaling.metadata import MetadataManager, NullMetadataManager
 from habitat_amd.analysis.wave_scaling.resimplified import resimplified_wave_scaling
 from habitat_amd.analysis.wave_scaling.roofline import roofline_wave_scaling
@@ -100,7 +101,12 @@ _ARGUMENTS = {"conv2d": conv2d_arguments, "linear": linear_arguments, "bmm": bmm
               "lstm": lstm_arguments}
 
 _BUILTIN = {unified_wave_scaling: "unified", roofline_wave_scaling: "roofline",
-            resimplified_wave_scaling: "resimplified"}
+            resimplified_wave_scaling: "resimplified", cdna_wave_scaling: "cdna"}
+
+
+def occupancy_device(device, mode):
+    """The description whose occupancy rules `mode` applies to `device`."""
+    return native_description(device) if mode == "cdna" else device
 
 
 def records_from_kernels(kernels, dest_device, metadata_manager, mode="unified", device=None):
@@ -226,7 +232,8 @@ class Predictor:
             kernels = [k for idx in idxs for k in run_times[idx].kernels]
             if kernels:
                 rec = records_from_kernels(kernels, dest_device, self._kernel_metadata, mode)
-                res = wave_scale(rec, origin, [dest_device], waves=False)
+                res = wave_scale(rec, occupancy_device(origin, mode),
+                                 [occupancy_device(dest_device, mode)], waves=False)
                 t = res.time_ns[0].cpu().numpy()
                 st = res.status[0].cpu().numpy()
                 bad = np.flatnonzero(st)

@@ -119,6 +119,7 @@ class SweepCall:
     reading anything back, so it can be repeated or captured in a HIP graph."""
 
     def __init__(self, plan, dests, device_features):
+        from habitat_amd.analysis import predictor as P
         self.plan = plan
         self.dests = dests
 
@@ -135,7 +136,8 @@ class SweepCall:
             whole = len(by_arch) == 1
             for idxs in by_arch.values():
                 rec = plan._records_for(dests[idxs[0]])
-                table = DeviceTable(plan.origin, [dests[i] for i in idxs])
+                table = DeviceTable(P.occupancy_device(plan.origin, plan.mode),
+                                    [P.occupancy_device(dests[i], plan.mode) for i in idxs])
                 at = None if whole else torch.tensor(idxs, device=plan.gpu)
                 self.groups.append((rec, table, at))
         self.dev_feats = None

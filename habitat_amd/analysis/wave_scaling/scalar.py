@@ -36,11 +36,12 @@ def raise_for_status(status):
     raise ZeroDivisionError("integer division or modulo by zero")
 
 
-def scale_one(kernel, origin_device, dest_device, metadata_manager, metrics):
+def scale_one(kernel, origin_device, dest_device, metadata_manager, metrics, lookup_device=None):
     """metrics: (eff, rd, wr) for the roofline strategy, None for the
-    no-metrics strategy.  Returns a PredictedKernel."""
+    no-metrics strategy.  `lookup_device`: the device the register table is
+    asked about when that is not `dest_device` itself.  Returns a PredictedKernel."""
     nb, block, dyn, stat, regs, t_ns = kernel_fields(kernel)
-    dest_regs = metadata_manager.kernel_registers_for(kernel, dest_device)
+    dest_regs = metadata_manager.kernel_registers_for(kernel, lookup_device or dest_device)
     dev = torch.device("cuda", torch.cuda.current_device())
     i32 = lambda v: torch.tensor([v], dtype=torch.int32, device=dev)
     f64 = lambda v: torch.tensor([v], dtype=torch.float64, device=dev)

@@ -117,10 +117,13 @@ int hbt_occupancy_host_model32_batch(const hbt_device_spec* spec, int64_t n,
   if (!hbt::occupancy_spec_in_domain(*spec)) return HBT_ESPEC;
   const hbt::OccDevice d = hbt::make_occ_device(*spec);
   if (!d.fast_ok()) return HBT_ESPEC;
-  for (int64_t i = 0; i < n; ++i)
-    out[i] = hbt::occupancy_fast(
-        d, block_size[i], hbt::smem_alloc(hbt::smem_sum(static_smem[i], dynamic_smem[i])),
-        regs[i] & 0xFFFF);
+  for (int64_t i = 0; i < n; ++i) {
+    const int32_t smem_total = hbt::smem_sum(static_smem[i], dynamic_smem[i]);
+    out[i] = (d.flags & hbt::kCdna)
+                 ? hbt::occupancy_cdna<false>(d, block_size[i], smem_total, regs[i] & 0xFFFF)
+                 : hbt::occupancy_fast(d, block_size[i], hbt::smem_alloc(smem_total),
+                                       regs[i] & 0xFFFF);
+  }
   return HBT_OK;
 }
 

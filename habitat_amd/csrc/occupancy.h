@@ -43,9 +43,10 @@ enum : uint32_t {
   kTuring = 1u << 4,     // cc 7.5: pool steps 32 KB/all
   kPoolSteps = 1u << 5,  // cc 7.x and a block's allocation can exceed pref_pool
   kWarpPow2 = 1u << 6,   // warp_size is a power of two: warp_shift is valid
+  kCdna = 1u << 7,       // AMD compute-unit model (HBT_COMPUTE_MAJOR_CDNA): occupancy_cdna
 };
 
-// Device-only constants of the occupancy model.  Every field fits 32 bits:
+// Device-only constants of the occupancy model (14 dwords).  Every field fits 32 bits:
 // hbt_device_spec_check bounds the shared-memory sizes below 2^31.
 struct OccDevice {
   uint32_t flags;
@@ -63,8 +64,17 @@ struct OccDevice {
   int32_t smem_per_sm;
   int32_t pref_pool;          // cc 7.x: the pool the default carve-out selects
 
+  // kCdna reuses two fields the compute-unit model has no other use for (the
+  // struct stays at 14 dwords of kernel-argument space and SGPRs per device):
+  // VGPRs per lane one SIMD holds (regs_per_sm / 4 / warp_size) ...
+  HBT_HD int32_t vgprs_per_simd() const { return regs_per_subpart4; }
+  // ... and the LDS allocation granule in bytes.
+  HBT_HD int32_t lds_granule() const { return regs_per_block; }
+
   HBT_HD bool ok() const { return (flags & kOk) != 0; }
   HBT_HD bool fast_ok() const { return (flags & kFastOk) != 0; }
+  // the kernels' lean instantiation: 32-bit arithmetic, NVIDIA rules only
+  HBT_HD bool lean_ok() const { return (flags & (kFastOk | kCdna)) == kFastOk; }
 };
 
 // Shared-memory pool a cc 7.x SM is configured to for an allocation of `size`
@@ -85,7 +95,8 @@ HBT_HD int32_t volta_pool(uint32_t flags, int32_t smem_per_sm, int32_t size) {
 inline OccDevice make_occ_device(const hbt_device_spec& s) {
   OccDevice d{};
   const int major = s.compute_major, minor = s.compute_minor;
-  const bool known = (major == 3 || major == 5 || major == 6 || major == 7);
+  const bool cdna = major == HBT_COMPUTE_MAJOR_CDNA;
+  const bool known = (major == 3 || major == 5 || major == 6 || major == 7 || cdna);
   const bool limits_ok = s.max_threads_per_block > 0 && s.max_threads_per_sm > 0 &&
                          s.regs_per_block > 0 && s.regs_per_sm > 0 && s.warp_size > 0 &&
                          s.smem_per_block != 0 && s.smem_per_sm != 0 && s.num_sms > 0;
@@ -115,13 +126,22 @@ inline OccDevice make_occ_device(const hbt_device_spec& s) {
   if (pow2) flags |= kWarpPow2;
   d.pref_pool = (major == 7) ? volta_pool(flags, d.smem_per_sm, d.smem_per_sm) : d.smem_per_sm;
   if (major == 7 && d.pref_pool < d.smem_per_block) flags |= kPoolSteps;
+  if (cdna) {
+    flags |= kCdna;
+    d.sub_shift = 2;    // 4 SIMDs per CU
+    d.block_slots = 16; // work-groups of more than one wave a CU holds (barrier resources)
+    d.regs_per_subpart4 = (s.regs_per_sm / 4) / d.warp_size;  // vgprs_per_simd()
+    d.regs_per_block = (minor == 5) ? 1280 : 512;             // lds_granule()
+  }
   // every division operand below 2^20 (so that dividend + divisor <= 2^21)
   const int32_t lim = 1 << 20;
-  const bool fast = !ok ||  // a rejected device needs no arithmetic at all
-                    (d.warp_size <= 1024 && d.max_threads_per_block < lim - 1024 &&
-                     d.max_warps_per_sm < lim && d.regs_per_subpart < lim &&
-                     d.smem_per_sm < lim && d.pref_pool < lim && d.smem_per_block < lim &&
-                     d.num_sms <= (1 << 14));
+  bool fast = !ok ||  // a rejected device needs no arithmetic at all
+              (d.warp_size <= 1024 && d.max_threads_per_block < lim - 1024 &&
+               d.max_warps_per_sm < lim && d.regs_per_subpart < lim &&
+               d.smem_per_sm < lim && d.pref_pool < lim && d.smem_per_block < lim &&
+               d.num_sms <= (1 << 14));
+  // LDS sizes are rounded up to the granule before they divide the CU's LDS
+  if (ok && cdna) fast = fast && d.smem_per_sm < lim / 2 && d.smem_per_block < lim / 2;
   if (fast) flags |= kFastOk;
   d.flags = flags;
   return d;
@@ -252,6 +272,60 @@ HBT_HD int32_t occupancy_fast(const OccDevice& d, int32_t block, const SmemAlloc
   return lim;
 }
 
+// Work-groups per compute unit on an AMD CDNA device (kCdna), after the
+// public occupancy rules of LLVM's AMDGPU backend (llvm/lib/Target/AMDGPU/Utils/
+// AMDGPUBaseInfo.cpp: getNumWavesPerEUWithNumVGPRs, getMaxWorkGroupsPerCU,
+// getLdsDwGranularity) for gfx90a and later, where a SIMD holds one unified file
+// of 512 VGPRs per lane allocated in granules of 8:
+//   waves per SIMD   = min(wave slots per SIMD, vgprs_per_simd / max(roundup(regs, 8), 8))
+//   by waves         = 4 * waves per SIMD / waves per work-group
+//   by work-group slots = all wave slots for one-wave work-groups, else 16
+//   by LDS           = smem_per_sm / roundup(bytes, granule), if any is used
+// and 0 for a launch the device cannot run (block size, registers per lane or
+// LDS per work-group beyond the limits, or a negative size).  There is no
+// counterpart in the reference.  `regs` is already narrowed to 16 bits.
+// EXACT_DIV: plain integer division (host; devices outside kFastOk).
+template <bool EXACT_DIV>
+HBT_HD int32_t occupancy_cdna(const OccDevice& d, int32_t block, int32_t smem_total, int32_t regs) {
+  if (!d.ok()) return 0;
+  const bool in_range = block > 0 && block <= d.max_threads_per_block &&
+                        regs <= d.vgprs_per_simd() && smem_total >= 0 &&
+                        smem_total <= d.smem_per_block;
+  block = in_range ? block : 1;
+  regs = in_range ? regs : 0;
+  const int32_t lds_bytes = in_range ? smem_total : 0;
+  const int32_t slots_per_simd = d.max_warps_per_sm >> 2;
+  int32_t alloc = (regs + 7) & ~7;
+  alloc = alloc < 8 ? 8 : alloc;
+  int32_t lim, lds, lim_lds;
+  if (EXACT_DIV) {
+    const int64_t waves = ((int64_t)block + d.warp_size - 1) / d.warp_size;
+    int64_t per_simd = d.vgprs_per_simd() / alloc;
+    per_simd = per_simd < slots_per_simd ? per_simd : slots_per_simd;
+    int64_t l = (per_simd * 4) / waves;
+    const int64_t group_slots = waves == 1 ? d.max_warps_per_sm : d.block_slots;
+    lim = (int32_t)(group_slots < l ? group_slots : l);
+    const int64_t rounded =
+        (((int64_t)lds_bytes + d.lds_granule() - 1) / d.lds_granule()) * d.lds_granule();
+    lds = rounded > 0 ? 1 : 0;
+    lim_lds = (int32_t)(d.smem_per_sm / (rounded > 0 ? rounded : 1));
+  } else {
+    const int32_t ws = d.warp_size;
+    const int32_t waves = (d.flags & kWarpPow2) ? ((block + ws - 1) >> d.warp_shift)
+                                                : fast_div(block + ws - 1, ws);
+    int32_t per_simd = fast_div(d.vgprs_per_simd(), alloc);
+    per_simd = per_simd < slots_per_simd ? per_simd : slots_per_simd;
+    lim = fast_div(per_simd << 2, waves);
+    const int32_t group_slots = waves == 1 ? d.max_warps_per_sm : d.block_slots;
+    lim = group_slots < lim ? group_slots : lim;
+    const int32_t granules = fast_div(lds_bytes + d.lds_granule() - 1, d.lds_granule());
+    lds = mul_small(granules, d.lds_granule());
+    lim_lds = fast_div(d.smem_per_sm, lds > 0 ? lds : 1);
+  }
+  lim = (lds > 0 && lim_lds < lim) ? lim_lds : lim;
+  return in_range ? lim : 0;
+}
+
 // The model without preconditions, in 64-bit arithmetic with C division (host,
 // and the kernel variant for devices outside kFastOk).  `regs` is already
 // narrowed to 16 bits; `smem_total` is smem_sum() of the two sizes.
@@ -315,7 +389,9 @@ HBT_HD int32_t occupancy_core(const OccDevice& d, int32_t block, int32_t smem_to
 // Host / slow-path occupancy: no preconditions.
 HBT_HD int32_t occupancy_exact(const OccDevice& d, int32_t block, int32_t dynamic_smem,
                                int32_t static_smem, int32_t regs) {
-  return occupancy_core(d, block, smem_sum(static_smem, dynamic_smem), (int32_t)(uint16_t)regs);
+  const int32_t smem_total = smem_sum(static_smem, dynamic_smem);
+  if (d.flags & kCdna) return occupancy_cdna<true>(d, block, smem_total, (int32_t)(uint16_t)regs);
+  return occupancy_core(d, block, smem_total, (int32_t)(uint16_t)regs);
 }
 
 }  // namespace hbt

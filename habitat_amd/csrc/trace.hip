@@ -36,7 +36,7 @@
 
 struct hbt_device_table {
   int32_t n_dest;
-  int32_t fast;            // every device (origin included) has kFastOk
+  int32_t fast;            // every device (origin included) has lean_ok()
   int device;
   hbt::OriginArgs origin;
   hbt::DestArgs* dests;    // device memory, [n_dest]
@@ -204,11 +204,11 @@ hbt_device_table* hbt_device_table_create(const hbt_device_spec* origin,
   t->n_dest = n_dest;
   t->device = device;
   t->origin = make_origin_args(*origin);
-  bool fast = t->origin.dev.fast_ok();
+  bool fast = t->origin.dev.lean_ok();
   std::vector<DestArgs> host((size_t)n_dest);
   for (int32_t d = 0; d < n_dest; ++d) {
     host[d] = make_dest_args(*origin, dests[d]);
-    fast = fast && host[d].dev.fast_ok();
+    fast = fast && host[d].dev.lean_ok();
   }
   t->fast = fast ? 1 : 0;
   t->dests = nullptr;

@@ -205,8 +205,8 @@ void launch(const WaveScaleArgs& args, hipStream_t stream) {
 
 hipError_t launch_wave_scale(const WaveScaleArgs& args, bool vectorised, hipStream_t stream) {
   if (args.n <= 0) return hipSuccess;
-  bool fast = args.origin.dev.fast_ok();
-  for (int d = 0; d < args.n_dest; ++d) fast = fast && args.dest[d].dev.fast_ok();
+  bool fast = args.origin.dev.lean_ok();
+  for (int d = 0; d < args.n_dest; ++d) fast = fast && args.dest[d].dev.lean_ok();
   if (vectorised) {
     if (fast) launch<kRecPerThread, true>(args, stream);
     else launch<kRecPerThread, false>(args, stream);

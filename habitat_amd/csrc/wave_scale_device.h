@@ -93,27 +93,35 @@ __device__ __forceinline__ double div_const(double x) {
 struct C100 { static constexpr double value = 100.0; };
 struct C1e9 { static constexpr double value = 1e9; };
 
-// FAST: every device of the launch has OccDevice::fast_ok, so the 32-bit model
-// applies to every record.  Otherwise the 64-bit model with real divisions runs
-// (devices with limits of 2^20 and more: not real hardware, but in the domain).
+// FAST: the lean instantiation.  Every device of the launch has
+// OccDevice::lean_ok, so the 32-bit NVIDIA-rule model applies to every record
+// and nothing else is compiled in.  Otherwise each device picks its model by
+// wave-uniform branches: the compute-unit model for AMD descriptions, the
+// 64-bit model with real divisions for devices with limits of 2^20 and more
+// (not real hardware, but in the domain).
 template <bool FAST>
 __device__ __forceinline__ int32_t occupancy_dev(const OccDevice& d, int32_t block,
                                                  int32_t smem_total, const SmemAlloc& sm,
                                                  int32_t regs) {
   regs &= 0xFFFF;  // uint16_t narrowing, cpp/src/cuda/kernel.h:108
   if (FAST) return occupancy_fast(d, block, sm, regs);
-  return occupancy_core(d, block, smem_total, regs);
+  if (d.flags & kCdna)
+    return d.fast_ok() ? occupancy_cdna<false>(d, block, smem_total, regs)
+                       : occupancy_cdna<true>(d, block, smem_total, regs);
+  return d.fast_ok() ? occupancy_fast(d, block, sm, regs)
+                     : occupancy_core(d, block, smem_total, regs);
 }
 
 // ceil(nb / sms) for 0 <= nb < 32 * sms.  The reference takes math.ceil of the
 // fp64 quotient (roofline.py:33-38); for operands below 2^53 that quotient is an
 // integer only when the division is exact, so the integer ceiling is the same.
-// On a fast_ok device sms <= 2^14 and nb < 2^19: float(nb) * (1/sms) is within
+// With sms <= 2^14 (every fast_ok device) nb < 2^19: float(nb) * (1/sms) is within
 // 2^-18 of the quotient, which is either an integer or at least 2^-14 away from
 // one, so ceil(product - 2^-16) is the exact ceiling.
 template <bool FAST>
 __device__ __forceinline__ int32_t ceil_div_small(int32_t nb, int32_t sms, float inv_sms) {
-  if (FAST) return (int32_t)ceilf(fmaf(__int2float_rn(nb), inv_sms, -0x1p-16f));
+  if (FAST || sms <= (1 << 14))
+    return (int32_t)ceilf(fmaf(__int2float_rn(nb), inv_sms, -0x1p-16f));
   return (int32_t)(((int64_t)nb + sms - 1) / sms);
 }
 

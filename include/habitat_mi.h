@@ -53,6 +53,24 @@ enum {
  * the host side.  The three double fields hold integer values, as the
  * reference's fields are integers (kernel.h:59-61).
  */
+/*
+ * compute_major of a device described by AMD's compute-unit model instead of
+ * the reference's NVIDIA one: 100 + the major HIP reports for the gfx9 family
+ * (compute_minor = HIP's minor: 0 gfx90a, 4 gfx942, 5 gfx950).  No counterpart
+ * in the reference, whose occupancy routine knows compute capabilities 3.x to
+ * 7.x and answers 0 for anything else (cpp/src/cuda/cuda_occupancy.h:573-694),
+ * plain 9.x included, which this library does too.  With this value the fields
+ * read: warp_size = wavefront size, max_threads_per_sm = wave slots of a CU x
+ * wavefront size, regs_per_sm = VGPRs of a CU counted per lane (4 SIMDs x 512
+ * x 64), smem_per_block / smem_per_sm = LDS a work-group may use / LDS of a
+ * CU, num_sms = CUs; regs_per_block is not used.  Occupancy (work-groups per
+ * CU) follows the public LLVM AMDGPU rules: VGPRs allocated in granules of 8
+ * per lane out of regs_per_sm / (4 x warp_size), a work-group's waves spread
+ * over the 4 SIMDs, 16 work-groups with more than one wave per CU, LDS in
+ * granules of 512 B (1280 B on gfx950).
+ */
+#define HBT_COMPUTE_MAJOR_CDNA 109
+
 typedef struct hbt_device_spec {
   int32_t compute_major, compute_minor;
   int32_t max_threads_per_block, max_threads_per_sm;
