@@ -112,6 +112,62 @@ def test_every_status_and_the_short_circuit(kat):
     assert list(st[:7]) == [1, 2, 0, 3, 3, 4, 0]
 
 
+def adversarial_records(n, seed):
+    """Every field drawn from a pool that mixes ordinary values with the ones a
+    formula mishandles first: zeros of both signs, subnormals, huge and tiny
+    magnitudes, infinities, NaN, negative and out-of-range integers."""
+    rng = np.random.default_rng(seed)
+    floats = np.array([0.0, -0.0, 5e-324, 1e-310, 2.3e-308, 1e-300, 1e-30, 1e-9, 0.5, 1.0, 37.5,
+                       100.0, 1e5, 1e9, 1e15, 1e100, 1e300, 1.7e308, np.inf, -np.inf, np.nan,
+                       -1.0, -1e-300, -1e9])
+    ints = np.array([0, 1, 2, 31, 32, 33, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 4096,
+                     49152, 49153, 65535, 65536, 65537, 98304, 1 << 20, (1 << 20) + 1, 1 << 24,
+                     (1 << 31) - 1, -(1 << 31), -1, -255, -256, -510, -511, -512])
+    pick_f = lambda ordinary: np.where(rng.random(n) < 0.6, ordinary, rng.choice(floats, n))
+    pick_i = lambda ordinary: np.where(rng.random(n) < 0.7, ordinary,
+                                       rng.choice(ints, n)).astype(np.int32)
+    return {
+        "num_blocks": pick_i(np.floor(2.0 ** rng.uniform(0, 20, n))),
+        "block_size": pick_i(rng.choice([64, 128, 256, 512, 1024], n)),
+        "dynamic_smem": pick_i(rng.integers(0, 30000, n)),
+        "static_smem": pick_i(rng.integers(0, 30000, n)),
+        "regs_per_thread": pick_i(rng.integers(16, 256, n)),
+        "dest_regs": np.where(rng.random(n) < 0.5, -1, pick_i(rng.integers(0, 300, n))).astype(np.int32),
+        "has_metrics": (rng.random(n) < 0.8).astype(np.uint8),
+        "run_time_ns": pick_f(np.floor(10.0 ** rng.uniform(3, 7, n))),
+        "flop_sp_efficiency": pick_f(10.0 ** rng.uniform(-2, 2, n)),
+        "dram_read_bytes": pick_f(np.floor(10.0 ** rng.uniform(3, 10, n))),
+        "dram_write_bytes": pick_f(np.floor(10.0 ** rng.uniform(3, 10, n))),
+    }
+
+
+def test_adversarial_field_values_agree_with_the_oracle_bit_for_bit_in_status():
+    """Statuses and integers exactly; times exactly where the oracle's is zero,
+    infinite or NaN, else within the tolerance."""
+    rec = adversarial_records(60_000, 99)
+    kr = KernelRecords.from_numpy(rec)
+    pairs = ((Device.V100, Device.MI355X), (Device.MI355X, Device.T4), (Device.P100, Device.V100))
+    for origin, dest in pairs:
+        out = wave_scale(kr, origin, [dest])
+        want = olib.wave_scale(odev(origin), odev(dest), rec)
+        assert np.array_equal(out.occ_origin.cpu().numpy(), want["occ_origin"])
+        assert np.array_equal(out.occ_dest[0].cpu().numpy(), want["occ_dest"])
+        assert np.array_equal(out.wave_dest[0].cpu().numpy(), want["wave_dest"])
+        st = out.status[0].cpu().numpy()
+        bad = np.flatnonzero(st != want["status"])
+        assert bad.size == 0, {k: v[bad[0]] for k, v in rec.items()}
+        assert len(set(st.tolist())) == 5           # every status occurs
+        t, w = out.time_ns[0].cpu().numpy(), want["time_ns"]
+        ok = st == 0
+        assert np.all(np.isnan(t[~ok]))
+        special = ok & ~(np.isfinite(w) & (w != 0))
+        assert special.sum() > 100
+        assert np.array_equal(t[special], w[special], equal_nan=True)
+        assert np.array_equal(np.signbit(t[special]), np.signbit(w[special]))
+        plain = ok & ~special
+        np.testing.assert_allclose(t[plain], w[plain], rtol=TIME_RTOL, atol=0)
+
+
 def test_golden_launch_configurations_on_all_fixture_devices(occupancy_golden):
     g, devices = occupancy_golden
     n = g["block"].shape[0]
