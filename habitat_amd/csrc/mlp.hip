@@ -238,6 +238,157 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
   }
 }
 
+// ---------------------------------------------------------------------------
+// Few rows (one prediction, the operations of one trace): one launch per layer.
+//
+// The fused kernel gives each workgroup 32 rows and the whole network, so a
+// batch of up to 32 rows runs on ONE compute unit, which has to pull all
+// 33.6 MB of weights through by itself (about 1 ms).  Here a layer is spread
+// over the chip instead: a workgroup takes NT n-tiles x one eighth of K x one
+// m-tile, its four waves split that K range again and add their 32 x 32
+// accumulators through LDS, and the eight K-partials of a layer are written to
+// a scratch buffer, [split][row][n].  They are summed, biased and rectified by
+// whoever reads them: the next layer's activation load, or the final dot
+// product.  The order of every sum is fixed, so results are reproducible.
+// Same packed weights, same MFMA instruction, same fragment layout as above.
+constexpr int kSplit = 8;            // K-partials per hidden layer
+constexpr int kSmallMaxRows = 512;   // largest batch that takes this path
+constexpr int kGroupsPerWave = (kWidth / 8) / kSplit / 4;  // 4 k-groups of a hidden layer
+static_assert(kGroupsPerWave == 4, "a wave of a hidden layer's workgroup owns four k-groups");
+
+struct LayerArgs {
+  const float* w_stream;   // packed weights, see above
+  int32_t groups_total;    // k-groups per wave stream (all layers)
+  int32_t g0;              // first stream group of this layer
+  int32_t kg;              // k-groups of this layer (K / 8)
+  int32_t splits;          // K-partials this launch writes (gridDim.y)
+  const float* p_in;       // [s_in][m_pad][kWidth], partials of the previous layer
+  int32_t s_in;
+  const float* bias_in;    // [kWidth], bias of the previous layer
+  const double* raw;       // FIRST: [n][in_features], with mu and sigma
+  const double* mu;
+  const double* sigma;
+  int32_t in_features;
+  int64_t n;
+  int32_t m_pad;           // rows rounded up to 32
+  float* p_out;            // [splits][m_pad][kWidth]
+};
+
+template <int NT, bool FIRST>
+__global__ __launch_bounds__(256) void mlp_layer_kernel(const LayerArgs a) {
+  __shared__ float red[4][NT][16][64];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 31, h = lane >> 5;
+  const int split = blockIdx.y;
+  const int64_t row = (int64_t)blockIdx.z * kRows + m;
+  const bool row_ok = row < a.n;
+
+  // this wave's k-groups: [first, first + count) of the layer's kg
+  const int per_split = a.kg / a.splits;
+  const int per_wave = (per_split + 3) / 4;
+  const int first = split * per_split + wave * per_wave;
+  int count = per_split - wave * per_wave;
+  count = count < 0 ? 0 : (count > per_wave ? per_wave : count);
+
+  f32x4 w[kGroupsPerWave][NT], x[kGroupsPerWave];
+#pragma unroll
+  for (int j = 0; j < kGroupsPerWave; ++j) {
+    const bool on = j < count;
+    const int gl = first + (on ? j : 0);  // layer-local group
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int tile = blockIdx.x * NT + t;               // n-tile of the layer, 0..31
+      const int owner = tile >> 3, slot = tile & 7;       // stream of the fused kernel's wave
+      const f32x4* p = reinterpret_cast<const f32x4*>(a.w_stream) +
+                       ((size_t)owner * a.groups_total + a.g0 + gl) * (8 * 64) + slot * 64 + lane;
+      w[j][t] = on ? *p : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    const int k = 8 * gl + 4 * h;
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (on && row_ok) {
+      if (FIRST) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (k + e < a.in_features)
+            v[e] = (float)((a.raw[row * a.in_features + k + e] - a.mu[k + e]) / a.sigma[k + e]);
+      } else {
+        v = *reinterpret_cast<const f32x4*>(a.bias_in + k);
+        for (int s = 0; s < a.s_in; ++s)
+          v += *reinterpret_cast<const f32x4*>(a.p_in + ((size_t)s * a.m_pad + row) * kWidth + k);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = fmaxf(v[e], 0.f);
+      }
+    }
+    x[j] = v;
+  }
+
+  f32x16 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+#pragma unroll
+  for (int j = 0; j < kGroupsPerWave; ++j)
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j][t][e], x[j][e], acc[t], 0, 0, 0);
+
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[wave][t][r][lane] = acc[t][r];
+  __syncthreads();
+  // thread (q = wave, lane) adds the four waves' registers 4q..4q+3: accumulator
+  // register 4g + e of lane (m, h) is output n = 8g + 4h + e of row m
+  const int q = wave;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    f32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      o[e] = ((red[0][t][4 * q + e][lane] + red[1][t][4 * q + e][lane]) +
+              red[2][t][4 * q + e][lane]) + red[3][t][4 * q + e][lane];
+    const int n0 = (blockIdx.x * NT + t) * 32 + 8 * q + 4 * h;
+    float* dst = a.p_out + ((size_t)split * a.m_pad + (size_t)blockIdx.z * kRows + m) * kWidth + n0;
+    *reinterpret_cast<f32x4*>(dst) = o;
+  }
+}
+
+struct LastArgs {
+  const float* p_in;     // [s_in][m_pad][kWidth]
+  int32_t s_in;
+  const float* bias_in;  // [kWidth]
+  const float* w_last;   // [kWidth]
+  float b_last;
+  int64_t n;
+  int32_t m_pad;
+  float* out;            // [n]
+};
+
+// fc2 for few rows: one wavefront per row.
+__global__ __launch_bounds__(256) void mlp_last_kernel(const LastArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.n) return;
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < kWidth / 256; ++i) {
+    const int k = 256 * i + 4 * lane;
+    f32x4 v = *reinterpret_cast<const f32x4*>(a.bias_in + k);
+    for (int s = 0; s < a.s_in; ++s)
+      v += *reinterpret_cast<const f32x4*>(a.p_in + ((size_t)s * a.m_pad + row) * kWidth + k);
+    const f32x4 wl = *reinterpret_cast<const f32x4*>(a.w_last + k);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum = fmaf(fmaxf(v[e], 0.f), wl[e], sum);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off);
+  if (lane == 0) a.out[row] = sum + a.b_last;
+}
+
 constexpr int kWaves = 4;  // one wave per SIMD: measured faster than two (fewer, longer MFMA runs between load bursts)
 constexpr size_t kLdsBytes =
     (size_t)(kRows * kStride + (kWaves * 64 / 32) * 32 + kWidth) * sizeof(float);
@@ -256,6 +407,7 @@ struct hbt_mlp {
   const float* bias;
   const float* w_last;
   float b_last;
+  float* scratch[2];   // few-rows path: two buffers of [kSplit][kSmallMaxRows][width] partials
 };
 
 namespace hbt {
@@ -325,11 +477,15 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
   const size_t off_stream = off; off = align_up(off + sizeof(float) * n_stream, 256);
   const size_t off_bias = off; off = align_up(off + sizeof(float) * n_bias, 256);
   const size_t off_last = off; off = align_up(off + sizeof(float) * kWidth, 256);
+  const size_t image = off;  // what is copied from the host; scratch follows
+  const size_t scratch_bytes = sizeof(float) * kSplit * kSmallMaxRows * kWidth;
+  const size_t off_scratch0 = off; off = align_up(off + scratch_bytes, 256);
+  const size_t off_scratch1 = off; off = align_up(off + scratch_bytes, 256);
   const size_t total = off;
 
   std::vector<unsigned char> host;
   try {
-    host.resize(total, 0);
+    host.resize(image, 0);
   } catch (const std::bad_alloc&) {
     *err = HBT_ENOMEM;
     return nullptr;
@@ -352,7 +508,7 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
     *err = HBT_ENOMEM;
     return nullptr;
   }
-  if (hipMemcpy(blob, host.data(), total, hipMemcpyHostToDevice) != hipSuccess) {
+  if (hipMemcpy(blob, host.data(), image, hipMemcpyHostToDevice) != hipSuccess) {
     (void)hipGetLastError();
     (void)hipFree(blob);
     *err = HBT_EHIP;
@@ -386,6 +542,8 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
   m->bias = reinterpret_cast<const float*>(base + off_bias);
   m->w_last = reinterpret_cast<const float*>(base + off_last);
   m->b_last = b[hidden_layers + 1][0];
+  m->scratch[0] = reinterpret_cast<float*>(base + off_scratch0);
+  m->scratch[1] = reinterpret_cast<float*>(base + off_scratch1);
   return m;
 }
 
@@ -407,6 +565,48 @@ int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* 
   }
   if (device != mlp->device) return HBT_EINVAL;
 
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  if (n <= kSmallMaxRows) {
+    // one launch per layer, K-partials through the handle's scratch buffers
+    const int m_tiles = (int)((n + kRows - 1) / kRows);
+    const int groups_total = mlp->in_padded / 8 + mlp->hidden * (kWidth / 8);
+    LayerArgs l{};
+    l.w_stream = mlp->w_stream;
+    l.groups_total = groups_total;
+    l.raw = raw_features; l.mu = mlp->mu; l.sigma = mlp->sigma;
+    l.in_features = mlp->in_features;
+    l.n = n;
+    l.m_pad = m_tiles * kRows;
+    const bool wide = m_tiles > 2;  // several n-tiles per workgroup once rows are re-read often
+    int s_in = 0;
+    const float* p_in = nullptr;
+    for (int layer = 0; layer <= mlp->hidden; ++layer) {
+      l.g0 = (layer == 0) ? 0 : mlp->in_padded / 8 + (layer - 1) * (kWidth / 8);
+      l.kg = (layer == 0) ? mlp->in_padded / 8 : kWidth / 8;
+      l.splits = (layer == 0) ? 1 : kSplit;
+      l.p_in = p_in; l.s_in = s_in;
+      l.bias_in = (layer == 0) ? nullptr : mlp->bias + (size_t)(layer - 1) * kWidth;
+      l.p_out = mlp->scratch[layer & 1];
+      const dim3 grid(wide ? 8 : 32, (unsigned)l.splits, (unsigned)m_tiles);
+      if (layer == 0) {
+        if (wide) hipLaunchKernelGGL((mlp_layer_kernel<4, true>), grid, dim3(256), 0, stream, l);
+        else hipLaunchKernelGGL((mlp_layer_kernel<1, true>), grid, dim3(256), 0, stream, l);
+      } else {
+        if (wide) hipLaunchKernelGGL((mlp_layer_kernel<4, false>), grid, dim3(256), 0, stream, l);
+        else hipLaunchKernelGGL((mlp_layer_kernel<1, false>), grid, dim3(256), 0, stream, l);
+      }
+      p_in = l.p_out;
+      s_in = l.splits;
+    }
+    LastArgs z{};
+    z.p_in = p_in; z.s_in = s_in;
+    z.bias_in = mlp->bias + (size_t)mlp->hidden * kWidth;
+    z.w_last = mlp->w_last; z.b_last = mlp->b_last;
+    z.n = n; z.m_pad = l.m_pad; z.out = out;
+    hipLaunchKernelGGL(mlp_last_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream, z);
+    return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
+  }
+
   MlpArgs a{};
   a.raw = raw_features;
   a.out = out;
@@ -421,7 +621,7 @@ int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* 
   a.w_last = mlp->w_last;
   a.b_last = mlp->b_last;
   hipLaunchKernelGGL(mlp_fused_kernel<kWaves>, dim3((unsigned)blocks), dim3(kWaves * 64),
-                     kLdsBytes, static_cast<hipStream_t>(hip_stream), a);
+                     kLdsBytes, stream, a);
   return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
 }
 

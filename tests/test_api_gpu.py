@@ -212,7 +212,9 @@ def test_device_sweep_matches_per_device_prediction():
         assert len(totals) == 24
         for i in (0, 7, 23):
             want = trace.to_device(devices[i], predictor).run_time_ms
-            assert totals[i] == pytest.approx(want, rel=1e-9)
+            # fp32 rounding in the MLP part: the sweep's 25 x 53 rows take the fused
+            # kernel, one device's 2 x 53 rows one launch per layer
+            assert totals[i] == pytest.approx(want, rel=1e-6)
         oracle_total = opred.trace_ms([oracle_operation_ms(op, devices[3], preds)
                                        for op in trace.operations])
         assert totals[3] == pytest.approx(oracle_total, rel=1e-5)

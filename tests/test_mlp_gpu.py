@@ -76,7 +76,9 @@ def test_trained_like_weights_with_wide_output_range():
     assert np.max(np.abs(y - y64)) <= 4 * np.max(np.abs(y32 - y64))
 
 
-@pytest.mark.parametrize("n", [1, 2, 31, 32, 33, 63, 65, 1000])
+# up to 512 rows run one launch per layer (two tile shapes: up to 64 rows, and
+# above), more rows the fused kernel
+@pytest.mark.parametrize("n", [1, 2, 31, 32, 33, 63, 64, 65, 96, 97, 511, 512, 513, 1000])
 def test_ragged_row_counts(n):
     rp = make("lstm")
     x, mu, sigma = synthetic.mlp_features("lstm", 1000, seed=5)
@@ -86,15 +88,32 @@ def test_ragged_row_counts(n):
     assert_close(y, omlp.forward_fp64(rp.model.state_dict(), x[:n], mu, sigma))
 
 
+def test_few_rows_path_and_fused_kernel_agree_on_the_same_rows():
+    """The same 300 rows alone (one launch per layer) and inside a batch of 900
+    (fused kernel): different summation orders, same answer to rounding."""
+    rp = make("conv2d")
+    x, mu, sigma = synthetic.mlp_features("conv2d", 900, seed=11)
+    rp.set_normalization(mu, sigma)
+    alone = rp.predict_batch(x[:300]).cpu().numpy()
+    inside = rp.predict_batch(x).cpu().numpy()[:300]
+    y64 = omlp.forward_fp64(rp.model.state_dict(), x[:300], mu, sigma)
+    assert_close(alone, y64)
+    assert_close(inside, y64)
+    assert np.max(np.abs(alone - inside)) <= 1e-5 * np.max(np.abs(y64))
+    # and the few-rows path is reproducible bit for bit
+    assert np.array_equal(alone, rp.predict_batch(x[:300]).cpu().numpy())
+
+
 def test_empty_batch():
     rp = make("bmm")
     rp.set_normalization(np.zeros(8), np.ones(8))
     assert rp.predict_batch(np.zeros((0, 8))).shape == (0,)
 
 
-def test_exact_cases_dead_relu_and_selector_weights():
+@pytest.mark.parametrize("rows", [40, 200, 700])
+def test_exact_cases_dead_relu_and_selector_weights(rows):
     rp = make("linear", hidden=2)
-    x, mu, sigma = synthetic.mlp_features("linear", 200, seed=6)
+    x, mu, sigma = synthetic.mlp_features("linear", rows, seed=6)
     rp.set_normalization(mu, sigma)
     with torch.no_grad():
         rp.model.mlp.layers[2].bias.fill_(-1e6)
@@ -121,7 +140,8 @@ def test_exact_cases_dead_relu_and_selector_weights():
         assert np.array_equal(y, want), pick
 
 
-def test_every_weight_position_is_wired():
+@pytest.mark.parametrize("rows", [33, 96, 640])
+def test_every_weight_position_is_wired(rows):
     # One hidden layer holding a random permutation matrix scaled by distinct
     # powers of two: out[r] = sum over units of 2^-(j%8) * in[perm[j]] exactly
     # representable, so a mis-packed weight shows up as a wrong value.
@@ -143,7 +163,7 @@ def test_every_weight_position_is_wired():
         rp.model.fc2.weight.copy_(torch.from_numpy(
             (rng.integers(0, 2, 1024) * 2 - 1).astype(np.float32))[None])
     rp.set_normalization(np.zeros(8), np.ones(8))
-    x = rng.integers(-4, 5, size=(96, 8)).astype(np.float64)   # small integers: exact sums
+    x = rng.integers(-4, 5, size=(rows, 8)).astype(np.float64)   # small integers: exact sums
     y = rp.predict_batch(x).cpu().numpy()
     y64 = omlp.forward_fp64(rp.model.state_dict(), x, np.zeros(8), np.ones(8))
     assert np.array_equal(y.astype(np.float64), y64)

@@ -178,9 +178,10 @@ def test_plan_reuse_and_subsets_agree_with_one_shot_sweep():
     again = plan.run(devices, feats).total_ms.cpu().numpy()
     np.testing.assert_array_equal(whole, again)
     part = plan.run(devices[5:9], feats).total_ms.cpu().numpy()
-    # a destination's total does not depend on which others share the launch;
-    # the MLP rows and the order of the fp64 atomic adds do, to rounding
-    np.testing.assert_allclose(part, whole[5:9], rtol=1e-12)
+    # a destination's total does not depend on which others share the launch,
+    # up to fp32 rounding in the MLP part: few rows take one launch per layer,
+    # many the fused kernel, and the two sum in different orders
+    np.testing.assert_allclose(part, whole[5:9], rtol=1e-6)
 
 
 def test_prepared_sweep_replays_in_a_hip_graph():
