@@ -373,6 +373,24 @@ def main():
                 "value": m / dt, "unit": "rows/s", "cores": threads, "kind": "port",
                 "sample": "oracle/mlp.py forward_fp32 (torch CPU fp32, one batched forward) on "
                           "the first %d rows, %d torch threads" % (m, threads)}
+        # few rows: the reference's own call pattern is one row per call (mlp.py:252-267)
+        few = {}
+        for rows in (1, 108, 512):
+            xs = xg[:rows].contiguous()
+            ys = torch.empty(rows, dtype=torch.float32, device="cuda")
+            _, f_launch = time_steps(lambda: rp.predict_batch(xs, out=ys), 50, 5)
+            few["rows_%d_us" % rows] = f_launch * 1e3
+        if not args.no_cpu:
+            from oracle import mlp as omlp
+            sd = rp.model.state_dict()
+            omlp.forward_fp32(sd, x[:1], mu, sigma)
+            t0 = time.perf_counter()
+            for i in range(20):
+                omlp.forward_fp32(sd, x[i:i + 1], mu, sigma)
+            few["cpu_rows_1_us"] = (time.perf_counter() - t0) / 20 * 1e6
+        few["note"] = ("up to 512 rows: one launch per layer over the whole GPU (mlp_layer_kernel); "
+                       "cpu_rows_1_us: torch CPU fp32, batch 1, as the reference predicts")
+        mlp["few_rows"] = few
         others = {}
         for other in [k for k in args.mlp_other_kinds.split(",") if k and k != kind]:
             torch.manual_seed(0)
