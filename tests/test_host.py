@@ -259,3 +259,27 @@ def test_csv_reports(tmp_path):
     assert p.endswith("resnet50+16-V100-e2e.csv")
     assert list(csv.reader(open(p))) == [["device", "run_time_ms"], ["V100", "5.75"], ["T4", "9.5"],
                                          ["P100", "7.25"]]
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU per box: `bench.py --gpus N` with N above 1 exits with a message."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2
+    assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_nothing_in_the_product_imports_the_oracle():
+    """The oracle is test infrastructure: the package must not reach for it."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    offenders = []
+    for base, _, files in os.walk(os.path.join(root, "habitat_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(base, f)).read()
+                if "oracle" in text.replace("oracle's", ""):
+                    offenders.append(os.path.join(base, f))
+    assert offenders == []
