@@ -274,7 +274,9 @@ struct LayerArgs {
   float* p_out;            // [splits][m_pad][kWidth]
 };
 
-template <int NT, bool FIRST>
+// S_IN: K-partials of the input (1 after fc1, kSplit after a hidden layer); a
+// compile-time count so that all of a lane's partial loads are in flight at once.
+template <int NT, bool FIRST, int S_IN>
 __global__ __launch_bounds__(256) void mlp_layer_kernel(const LayerArgs a) {
   __shared__ float red[4][NT][16][64];
   const int tid = threadIdx.x;
@@ -313,9 +315,13 @@ __global__ __launch_bounds__(256) void mlp_layer_kernel(const LayerArgs a) {
           if (k + e < a.in_features)
             v[e] = (float)((a.raw[row * a.in_features + k + e] - a.mu[k + e]) / a.sigma[k + e]);
       } else {
+        f32x4 part[S_IN];
+#pragma unroll
+        for (int s = 0; s < S_IN; ++s)
+          part[s] = *reinterpret_cast<const f32x4*>(a.p_in + ((size_t)s * a.m_pad + row) * kWidth + k);
         v = *reinterpret_cast<const f32x4*>(a.bias_in + k);
-        for (int s = 0; s < a.s_in; ++s)
-          v += *reinterpret_cast<const f32x4*>(a.p_in + ((size_t)s * a.m_pad + row) * kWidth + k);
+#pragma unroll
+        for (int s = 0; s < S_IN; ++s) v += part[s];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = fmaxf(v[e], 0.f);
       }
@@ -369,17 +375,25 @@ struct LastArgs {
 };
 
 // fc2 for few rows: one wavefront per row.
+template <int S_IN>
 __global__ __launch_bounds__(256) void mlp_last_kernel(const LastArgs a) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= a.n) return;
+  f32x4 part[kWidth / 256][S_IN];
+#pragma unroll
+  for (int i = 0; i < kWidth / 256; ++i)
+#pragma unroll
+    for (int s = 0; s < S_IN; ++s)
+      part[i][s] = *reinterpret_cast<const f32x4*>(
+          a.p_in + ((size_t)s * a.m_pad + row) * kWidth + 256 * i + 4 * lane);
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < kWidth / 256; ++i) {
     const int k = 256 * i + 4 * lane;
     f32x4 v = *reinterpret_cast<const f32x4*>(a.bias_in + k);
-    for (int s = 0; s < a.s_in; ++s)
-      v += *reinterpret_cast<const f32x4*>(a.p_in + ((size_t)s * a.m_pad + row) * kWidth + k);
+#pragma unroll
+    for (int s = 0; s < S_IN; ++s) v += part[i][s];
     const f32x4 wl = *reinterpret_cast<const f32x4*>(a.w_last + k);
 #pragma unroll
     for (int e = 0; e < 4; ++e) sum = fmaf(fmaxf(v[e], 0.f), wl[e], sum);
@@ -589,11 +603,16 @@ int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* 
       l.p_out = mlp->scratch[layer & 1];
       const dim3 grid(wide ? 8 : 32, (unsigned)l.splits, (unsigned)m_tiles);
       if (layer == 0) {
-        if (wide) hipLaunchKernelGGL((mlp_layer_kernel<4, true>), grid, dim3(256), 0, stream, l);
-        else hipLaunchKernelGGL((mlp_layer_kernel<1, true>), grid, dim3(256), 0, stream, l);
+        if (wide) hipLaunchKernelGGL((mlp_layer_kernel<4, true, 1>), grid, dim3(256), 0, stream, l);
+        else hipLaunchKernelGGL((mlp_layer_kernel<1, true, 1>), grid, dim3(256), 0, stream, l);
+      } else if (s_in == 1) {
+        if (wide) hipLaunchKernelGGL((mlp_layer_kernel<4, false, 1>), grid, dim3(256), 0, stream, l);
+        else hipLaunchKernelGGL((mlp_layer_kernel<1, false, 1>), grid, dim3(256), 0, stream, l);
       } else {
-        if (wide) hipLaunchKernelGGL((mlp_layer_kernel<4, false>), grid, dim3(256), 0, stream, l);
-        else hipLaunchKernelGGL((mlp_layer_kernel<1, false>), grid, dim3(256), 0, stream, l);
+        if (wide)
+          hipLaunchKernelGGL((mlp_layer_kernel<4, false, kSplit>), grid, dim3(256), 0, stream, l);
+        else
+          hipLaunchKernelGGL((mlp_layer_kernel<1, false, kSplit>), grid, dim3(256), 0, stream, l);
       }
       p_in = l.p_out;
       s_in = l.splits;
@@ -603,7 +622,9 @@ int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* 
     z.bias_in = mlp->bias + (size_t)mlp->hidden * kWidth;
     z.w_last = mlp->w_last; z.b_last = mlp->b_last;
     z.n = n; z.m_pad = l.m_pad; z.out = out;
-    hipLaunchKernelGGL(mlp_last_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream, z);
+    const dim3 rows_grid((unsigned)((n + 3) / 4));
+    if (s_in == 1) hipLaunchKernelGGL(mlp_last_kernel<1>, rows_grid, dim3(256), 0, stream, z);
+    else hipLaunchKernelGGL(mlp_last_kernel<kSplit>, rows_grid, dim3(256), 0, stream, z);
     return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
   }
 
