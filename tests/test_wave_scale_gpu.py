@@ -168,6 +168,55 @@ def test_adversarial_field_values_agree_with_the_oracle_bit_for_bit_in_status():
         np.testing.assert_allclose(t[plain], w[plain], rtol=TIME_RTOL, atol=0)
 
 
+def test_more_than_2_to_28_records_take_64_bit_offsets():
+    """Above 2^28 records byte offsets no longer fit 32 bits and the kernel's
+    64-bit-offset instantiation runs.  Records are generated on the GPU (19 GB of
+    columns); a sample from the start, the 32-bit boundary and the ragged end
+    is checked against the oracle."""
+    n = (1 << 28) + 12345
+    free, _ = torch.cuda.mem_get_info()
+    if free < 40 * (1 << 30):
+        pytest.skip("needs 40 GB of free device memory")
+    g = torch.Generator(device="cuda").manual_seed(5)
+    ri = lambda lo, hi: torch.randint(lo, hi, (n,), generator=g, device="cuda", dtype=torch.int32)
+    cols = {
+        "num_blocks": ri(1, 1 << 20),
+        "block_size": ri(1, 9) * 128,
+        "dynamic_smem": ri(0, 20000), "static_smem": ri(0, 20000),
+        "regs_per_thread": ri(16, 129),
+    }
+    for name, lo, hi in (("run_time_ns", 3.0, 7.0), ("flop_sp_efficiency", -2.0, 2.0),
+                         ("dram_read_bytes", 3.0, 10.0), ("dram_write_bytes", 3.0, 10.0)):
+        u = torch.rand((n,), generator=g, device="cuda", dtype=torch.float64)
+        cols[name] = torch.floor(10.0 ** (lo + (hi - lo) * u)) if name != "flop_sp_efficiency" \
+            else 10.0 ** (lo + (hi - lo) * u)
+        del u
+    kr = KernelRecords(cols)
+    out = WaveScaleOutput(n, 1, kr.device, waves=False, status=True)
+    # poison the outputs so that a record the kernel skipped shows
+    out.time_ns.fill_(-7.0)
+    out.occ_dest.fill_(-7)
+    wave_scale(kr, Device.V100, [Device.MI355X], out=out)
+    torch.cuda.synchronize()
+    boundary = 1 << 28
+    idx = torch.cat([torch.arange(0, 2000), torch.arange(boundary - 2000, boundary + 2000),
+                     torch.arange(n - 2000, n),
+                     torch.randint(0, n, (20000,), generator=torch.Generator().manual_seed(6))]).cuda()
+    rec = {k: v[idx].cpu().numpy() for k, v in cols.items()}
+    want = olib.wave_scale(odev(Device.V100), odev(Device.MI355X), rec)
+    assert np.array_equal(out.occ_origin[idx].cpu().numpy(), want["occ_origin"])
+    assert np.array_equal(out.occ_dest[0][idx].cpu().numpy(), want["occ_dest"])
+    st = out.status[0][idx].cpu().numpy()
+    assert np.array_equal(st, want["status"])
+    t = out.time_ns[0][idx].cpu().numpy()
+    ok = st == 0
+    assert ok.sum() > 10000
+    np.testing.assert_allclose(t[ok], want["time_ns"][ok], rtol=TIME_RTOL, atol=0)
+    # every record was written: no poison left anywhere
+    assert int((out.occ_dest == -7).sum().item()) == 0
+    assert int((out.time_ns == -7.0).sum().item()) == 0
+
+
 def test_golden_launch_configurations_on_all_fixture_devices(occupancy_golden):
     g, devices = occupancy_golden
     n = g["block"].shape[0]
