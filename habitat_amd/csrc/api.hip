@@ -121,7 +121,7 @@ int hbt_occupancy_host_model32_batch(const hbt_device_spec* spec, int64_t n,
     const int32_t smem_total = hbt::smem_sum(static_smem[i], dynamic_smem[i]);
     out[i] = (d.flags & hbt::kCdna)
                  ? hbt::occupancy_cdna<false>(d, block_size[i], smem_total, regs[i] & 0xFFFF)
-                 : hbt::occupancy_fast(d, block_size[i], hbt::smem_alloc(smem_total),
+                 : hbt::occupancy_fast<false>(d, block_size[i], hbt::smem_alloc(smem_total),
                                        regs[i] & 0xFFFF);
   }
   return HBT_OK;

@@ -73,8 +73,13 @@ struct OccDevice {
 
   HBT_HD bool ok() const { return (flags & kOk) != 0; }
   HBT_HD bool fast_ok() const { return (flags & kFastOk) != 0; }
-  // the kernels' lean instantiation: 32-bit arithmetic, NVIDIA rules only
-  HBT_HD bool lean_ok() const { return (flags & (kFastOk | kCdna)) == kFastOk; }
+  // the kernels' lean instantiation: an accepted NVIDIA-rule device whose
+  // model is straight-line code in 32-bit arithmetic (power-of-two warp size,
+  // no cc 6.0 re-check, no cc 7.x pool steps)
+  HBT_HD bool lean_ok() const {
+    return (flags & (kOk | kFastOk | kWarpPow2 | kCdna | kGp100 | kPoolSteps)) ==
+           (kOk | kFastOk | kWarpPow2);
+  }
 };
 
 // Shared-memory pool a cc 7.x SM is configured to for an allocation of `size`
@@ -220,17 +225,22 @@ HBT_HD SmemAlloc smem_alloc(int32_t smem_total) {
 // budget is zeroed.  Branches on device constants are wave-uniform.  The
 // register and warp-slot limits share their divisor, and floor division is
 // monotonic, so min(floor(a / w), floor(b / w)) is taken as floor(min(a, b) / w).
+//
+// LEAN: the device has lean_ok(), so none of the wave-uniform branches is
+// compiled in and the whole model is one basic block (the kernel then
+// interleaves the arithmetic of a thread's records).
+template <bool LEAN = false>
 HBT_HD int32_t occupancy_fast(const OccDevice& d, int32_t block, const SmemAlloc& sm,
                               int32_t regs) {
-  if (!d.ok()) return 0;
+  if (!LEAN && !d.ok()) return 0;
   // regs <= 256 is the per-thread limit; it also keeps regs * warp_size below 2^19
   const bool in_range = block > 0 && block <= d.max_threads_per_block && regs <= 256;
   block = in_range ? block : 1;
   regs = in_range ? regs : 0;
 
   const int32_t ws = d.warp_size;
-  const int32_t warps = (d.flags & kWarpPow2) ? ((block + ws - 1) >> d.warp_shift)
-                                              : fast_div(block + ws - 1, ws);
+  const int32_t warps = (LEAN || (d.flags & kWarpPow2)) ? ((block + ws - 1) >> d.warp_shift)
+                                                      : fast_div(block + ws - 1, ws);
   const float rcp_warps = fast_rcp(warps);
 
   // registers: 256 per-warp granularity, allocated per sub-partition; a block
@@ -247,7 +257,7 @@ HBT_HD int32_t occupancy_fast(const OccDevice& d, int32_t block, const SmemAlloc
   const int32_t per_warp1 = per_warp > 0 ? per_warp : 1;
   const float rcp_per_warp = fast_rcp(per_warp1);
   const int32_t reg_warps = fast_div_r(d.regs_per_subpart, per_warp1, rcp_per_warp) << d.sub_shift;
-  if (d.flags & kGp100) {
+  if (!LEAN && (d.flags & kGp100)) {
     // cc 6.0 must also fit a 4-sub-partition Pascal SM
     const int32_t warps_up4 = (warps + 3) & ~3;
     fits = fits && mul_small(per_warp256, warps_up4) <= block_regs256 &&
@@ -262,7 +272,7 @@ HBT_HD int32_t occupancy_fast(const OccDevice& d, int32_t block, const SmemAlloc
 
   // shared memory: an allocation above the per-block limit leaves no pool
   int32_t pool = d.pref_pool;
-  if (d.flags & kPoolSteps) {
+  if (!LEAN && (d.flags & kPoolSteps)) {
     const int32_t stepped = volta_pool(d.flags, d.smem_per_sm, sm.alloc);
     pool = pool < sm.alloc ? stepped : pool;
   }

@@ -102,7 +102,9 @@ __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a)
   // lanes past the end form a run of their own so that they never swallow a tail
   const int32_t seg = in_range ? (a.segment != nullptr ? a.segment[j] : 0) : -1;
 
-  const RecordMid m = origin_part<FAST>(a.origin, r);
+  RecordMid m = origin_part<FAST>(a.origin, r);
+  if (__builtin_expect(m.redo_gflops, 0))
+    m.num_gflops = origin_gflops_exact(a.origin.peak_gflops, r.eff, r.t);
   const RecordOut o = dest_part<FAST, false>(p, r, m, 0.0);
 
   const bool ok = in_range && o.status == HBT_ST_OK;

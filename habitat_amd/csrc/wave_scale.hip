@@ -128,6 +128,15 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
                       true, t[k], eff[k], rd[k], wr[k]};
     mid[k] = origin_part<FAST>(a.origin, rin[k]);
   }
+  bool redo = false;
+#pragma unroll
+  for (int k = 0; k < R; ++k) redo = redo || mid[k].redo_gflops;
+  if (__builtin_expect(redo, 0)) {
+#pragma unroll
+    for (int k = 0; k < R; ++k)
+      if (mid[k].redo_gflops)
+        mid[k].num_gflops = origin_gflops_exact(a.origin.peak_gflops, rin[k].eff, rin[k].t);
+  }
   // Opaque to the optimiser: keeps the unpacking of the flags from moving up
   // to the load.
   asm volatile("" : "+v"(hm_bits));

@@ -48,6 +48,7 @@ struct RecordMid {
   int32_t occ_o, wave_o;
   int32_t origin_max_occ;  // ceil(num_blocks / origin.num_sms) when small_o, else 0
   bool small_o;            // num_blocks // origin_wave == 0
+  bool redo_gflops;        // num_gflops needs origin_gflops_exact (see div_const)
   double num_gflops, total_gb;
 };
 
@@ -78,17 +79,21 @@ __device__ __forceinline__ double exp2_poly(double x) {
 // division it replaces: q = x * (1/c) is within an ulp of the quotient, the
 // remainder x - q*c is exact in an FMA, and adding remainder * (1/c) back
 // rounds to the nearest double (Markstein's correction; checked against `/`
-// on 4e8 operands for each constant used here).  Operands whose remainder
-// could underflow or overflow take the hardware sequence instead.
+// on 4e8 operands for each constant used here).  Valid where div_const_safe
+// holds; elsewhere the remainder could underflow or overflow and the caller
+// must divide for real.
 template <class C>
 __device__ __forceinline__ double div_const(double x) {
   constexpr double c = C::value, rc = 1.0 / C::value;
-  // safe: zero, or finite with |x| >= 2^-900 (c > 1, so nothing can overflow)
-  const double ax = fabs(x);
-  if (__builtin_expect(!((ax >= 0x1p-900 && ax < __builtin_inf()) || ax == 0.0), 0)) return x / c;
   const double q = x * rc;
   const double r = fma(-q, c, x);
   return fma(r, rc, q);
+}
+
+// zero, or finite with |x| >= 2^-900 (c > 1, so nothing can overflow)
+__device__ __forceinline__ bool div_const_safe(double x) {
+  const double ax = fabs(x);
+  return (ax >= 0x1p-900 && ax < __builtin_inf()) || ax == 0.0;
 }
 struct C100 { static constexpr double value = 100.0; };
 struct C1e9 { static constexpr double value = 1e9; };
@@ -104,7 +109,7 @@ __device__ __forceinline__ int32_t occupancy_dev(const OccDevice& d, int32_t blo
                                                  int32_t smem_total, const SmemAlloc& sm,
                                                  int32_t regs) {
   regs &= 0xFFFF;  // uint16_t narrowing, cpp/src/cuda/kernel.h:108
-  if (FAST) return occupancy_fast(d, block, sm, regs);
+  if (FAST) return occupancy_fast<true>(d, block, sm, regs);
   if (d.flags & kCdna)
     return d.fast_ok() ? occupancy_cdna<false>(d, block, smem_total, regs)
                        : occupancy_cdna<true>(d, block, smem_total, regs);
@@ -140,9 +145,22 @@ __device__ __forceinline__ RecordMid origin_part(const OriginArgs& o, const Reco
   // total_gb reach no output: gamma is then forced to 1 by num_gflops < 1e-9
   // or lies within 1e-290 of 0.)
   m.total_gb = (r.rd + r.wr) * 0x1p-30;
+  // eff / 100 * peak * t / 1e9 with the two constant divisions as corrected
+  // multiplications.  No branch here: the caller tests redo_gflops of all its
+  // records at once, so that their arithmetic stays in one basic block.
   const double gflops_per_second = div_const<C100>(r.eff) * o.peak_gflops;
-  m.num_gflops = div_const<C1e9>(gflops_per_second * r.t);
+  const double scaled = gflops_per_second * r.t;
+  m.num_gflops = div_const<C1e9>(scaled);
+  m.redo_gflops = !(div_const_safe(r.eff) && div_const_safe(scaled));
   return m;
+}
+
+// The same quantity with the divisions the reference performs (roofline.py:73-76),
+// for records whose operands div_const cannot take: infinities, NaN, magnitudes
+// below 2^-900.
+__device__ __noinline__ double origin_gflops_exact(double peak_gflops, double eff, double t) {
+  const double gflops_per_second = eff / 100 * peak_gflops;
+  return gflops_per_second * t / 1e9;
 }
 
 struct RecordOut {
@@ -209,8 +227,11 @@ __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn
   const double gamma_compl = 1.0 - gamma;
   const double log2_small = p.log2_clk + log2_count<PERMUTE>(log2_lane, dest_max_occ) -
                             log2_count<PERMUTE>(log2_lane, m.origin_max_occ);
-  const double exponent =
-      small ? gamma_compl * log2_small : gamma * p.log2_bw + gamma_compl * p.log2_clk_sm;
+  // small: (1-gamma) * log2_small; else gamma * L_bw + (1-gamma) * L_clk_sm.  As one
+  // expression with selected operands (a zero first term is exact), so that
+  // the code stays free of branches.
+  const double exponent = (small ? 0.0 : gamma) * p.log2_bw +
+                          gamma_compl * (small ? log2_small : p.log2_clk_sm);
   const double t = r.t * exp2_poly(exponent);
   o.t = (status == HBT_ST_OK) ? t : __builtin_nan("");
   return o;
