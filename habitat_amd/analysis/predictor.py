@@ -6,6 +6,7 @@ The reference predicts one kernel and one operation at a time.  Here
 `predict_trace_times` gather every kernel record (resp. every MLP feature row)
 of a trace and hand them to the GPU in one call each.
 """
+import collections
 import functools
 import logging
 import operator
@@ -139,6 +140,8 @@ def records_from_kernels(kernels, dest_device, metadata_manager, mode="unified",
 
 
 class Predictor:
+    _RECORD_CACHE_SETS = 8
+
     def __init__(self, kernel_metadata_file=None, wave_scaling_strategy=unified_wave_scaling,
                  mlp_predictors=None):
         """`kernel_metadata_file`: sqlite register table (default: data/kernels.sqlite
@@ -153,6 +156,7 @@ class Predictor:
         else:
             self._kernel_metadata = NullMetadataManager()
         self._wave_scaling_strategy = wave_scaling_strategy
+        self._record_cache = collections.OrderedDict()
 
         mlp_predictors = dict(mlp_predictors or {})
         for kind in _MLP_KINDS:
@@ -231,7 +235,8 @@ class Predictor:
         for origin, idxs in by_origin.values():
             kernels = [k for idx in idxs for k in run_times[idx].kernels]
             if kernels:
-                rec = records_from_kernels(kernels, dest_device, self._kernel_metadata, mode)
+                rec = self._records_of([run_times[idx] for idx in idxs], kernels, dest_device,
+                                       mode)
                 res = wave_scale(rec, occupancy_device(origin, mode),
                                  [occupancy_device(dest_device, mode)], waves=False)
                 t = res.time_ns[0].cpu().numpy()
@@ -252,6 +257,30 @@ class Predictor:
             preds = [PredictedKernel(k, v) for k, v in zip(rt.kernels, vals)]
             out.append(self._assemble(rt, preds, dest_device))
         return out
+
+    def _records_of(self, passes, kernels, dest_device, mode):
+        """The kernel records of `passes` as columns on the GPU.  The last few
+        sets are kept (keyed by the identity of the measured passes, which this
+        package treats as immutable once measured), so that predicting one trace
+        for one destination after another converts and uploads its kernels once.
+        The register column depends on the destination's architecture only."""
+        lut = not isinstance(self._kernel_metadata, NullMetadataManager)
+        key = (tuple(id(p) for p in passes), mode, dest_device.compute_capability if lut else None,
+               torch.cuda.current_device())
+        hit = self._record_cache.get(key)
+        if hit is not None:
+            self._record_cache.move_to_end(key)
+            return hit[0]
+        rec = records_from_kernels(kernels, dest_device, self._kernel_metadata, mode)
+        self._record_cache[key] = (rec, list(passes))   # the passes stay alive with their ids
+        while len(self._record_cache) > self._RECORD_CACHE_SETS:
+            self._record_cache.popitem(last=False)
+        return rec
+
+    def clear_record_cache(self):
+        """Forget the cached kernel-record columns (after changing a measured
+        kernel in place)."""
+        self._record_cache.clear()
 
     @staticmethod
     def _assemble(run_time, predicted_kernels, dest_device):
