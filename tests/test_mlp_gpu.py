@@ -188,12 +188,14 @@ def test_scalar_predict_and_checkpoint_round_trip(tmp_path):
         RuntimePredictor("conv2d", 8, 1024).predict(args, "V100")     # no mu/sigma
 
 
-def test_config2_full_size_properties():
-    # 1M rows: the oracle is too slow for all of them, so check a strided
-    # sample against it and, over the whole batch, invariance to row order.
-    rp = make("conv2d")
+@pytest.mark.parametrize("kind", ["conv2d", "linear", "bmm", "lstm"])
+def test_config2_and_config3_full_size_properties(kind):
+    # 1M rows (configs[2]: conv2d; configs[3]: the other three): the oracle is
+    # too slow for all of them, so check a strided sample against it and, over
+    # the whole batch, invariance to row order.
+    rp = make(kind)
     n = 1_000_000
-    x, mu, sigma = synthetic.mlp_features("conv2d", n, seed=2)
+    x, mu, sigma = synthetic.mlp_features(kind, n, seed=2)
     rp.set_normalization(mu, sigma)
     xg = torch.from_numpy(x).cuda()
     y = rp.predict_batch(xg)
