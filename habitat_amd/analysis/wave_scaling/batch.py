@@ -90,6 +90,24 @@ class WaveScaleOutput:
                           if waves else None)
         self.status = torch.empty((n_dest, n), dtype=torch.uint8, device=device) if status else None
 
+    def wave_counts(self, num_blocks):
+        """(origin [n], destination [n_dest, n]) int64 tensors of
+        `num_blocks // wave_size`, the quotient the reference compares with zero
+        to tell a kernel that fits one wave (wave_scaling/roofline.py:29-30),
+        with Python's floor semantics; -1 where the wave size is 0 (the
+        reference raises ZeroDivisionError there).  Needs the wave-size outputs."""
+        if self.wave_origin is None:
+            raise ValueError("allocate the output with waves=True")
+        nb = num_blocks.to(torch.int64)
+
+        def quotient(wave):
+            wave = wave.to(torch.int64)
+            safe = torch.where(wave == 0, torch.ones_like(wave), wave)
+            q = torch.div(nb.expand_as(wave), safe, rounding_mode="floor")
+            return torch.where(wave == 0, torch.full_like(q, -1), q)
+
+        return quotient(self.wave_origin), quotient(self.wave_dest)
+
 
 def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else None

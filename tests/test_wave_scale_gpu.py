@@ -268,6 +268,22 @@ def test_ragged_sizes_single_and_multi_destination(n):
     check(rec, Device.V100, dests, wave_scale(kr, Device.V100, dests))
 
 
+def test_wave_counts_are_the_reference_quotients():
+    rec = adversarial_records(5000, 17)
+    kr = KernelRecords.from_numpy(rec)
+    dests = [Device.MI355X, Device.T4]
+    out = wave_scale(kr, Device.V100, dests)
+    count_o, count_d = out.wave_counts(kr.columns["num_blocks"])
+    wave_o = out.wave_origin.cpu().numpy().astype(object)
+    nb = rec["num_blocks"].astype(object)
+    want_o = [int(b) // int(w) if w else -1 for b, w in zip(nb, wave_o)]
+    assert count_o.cpu().tolist() == want_o
+    for di in range(2):
+        wave_d = out.wave_dest[di].cpu().numpy().astype(object)
+        assert count_d[di].cpu().tolist() == [int(b) // int(w) if w else -1
+                                              for b, w in zip(nb, wave_d)]
+
+
 def test_empty_input_and_no_destinations():
     rec, _ = synthetic.kernel_records(8, Device.V100, seed=0)
     empty = {k: v[:0] for k, v in rec.items()}
