@@ -37,6 +37,7 @@ logger = logging.getLogger(__name__)
 CONV2D_PARAMS = ["input", "weight", "bias", "stride", "padding", "dilation", "groups"]
 LINEAR_PARAMS = ["input", "weight", "bias"]
 BMM_PARAMS = ["input", "mat2", "out"]
+MATMUL_PARAMS = ["input", "other", "out"]   # defined and unused in the reference too (predictor.py:50)
 LSTM_PARAMS_NO_BATCH_SIZES = ["input", "hx", "flat_weights", "bias", "num_layers", "dropout",
                               "training", "bidirectional", "batch_first"]
 LSTM_PARAMS = ["input", "batch_sizes", "hx", "flat_weights", "bias", "num_layers", "dropout",

@@ -7,8 +7,16 @@ predictor is built on first use.
 from habitat_amd.analysis.predictor import Predictor
 
 
+class _LazyDefaultPredictor:
+    """`Trace.DefaultPredictor` (analysis/trace.py:11), built when first read."""
+
+    def __get__(self, instance, owner):
+        return owner.default_predictor()
+
+
 class Trace:
     _default_predictor = None
+    DefaultPredictor = _LazyDefaultPredictor()
 
     def __init__(self, device, operations):
         self._device = device

@@ -223,3 +223,20 @@ def ratio_scale(pred, run_time_ms, n_dest, totals=None, want_ms=True, stream=Non
                                         ctypes.c_void_p(stream.cuda_stream))
     _lib.check(rc, "hbt_ratio_scale")
     return out
+
+
+def roofline_gamma(records, origin, dest, stream=None):
+    """The roofline exponent of every record (see hbt_roofline_gamma): a float64
+    GPU tensor [n], NaN where the reference's assertion on gamma fails.  Every
+    record is taken to have its metrics."""
+    out = torch.empty((records.n,), dtype=torch.float64, device=records.device)
+    if stream is None:
+        stream = torch.cuda.current_stream(records.device)
+    c = records.columns
+    with torch.cuda.device(records.device):
+        rc = _lib.lib().hbt_roofline_gamma(
+            ctypes.byref(origin.spec), ctypes.byref(dest.spec), records.n,
+            _ptr(c["run_time_ns"]), _ptr(c["flop_sp_efficiency"]), _ptr(c["dram_read_bytes"]),
+            _ptr(c["dram_write_bytes"]), _ptr(out), ctypes.c_void_p(stream.cuda_stream))
+    _lib.check(rc, "hbt_roofline_gamma")
+    return out

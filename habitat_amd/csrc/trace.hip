@@ -132,6 +132,32 @@ __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a)
     unsafeAtomicAdd(a.out_sum + (int64_t)d * a.n_segments + seg, v);
 }
 
+struct GammaArgs {
+  int64_t n;
+  const double* run_time_ns;
+  const double* flop_sp_efficiency;
+  const double* dram_read_bytes;
+  const double* dram_write_bytes;
+  double* out_gamma;
+  double peak_gflops;   // origin
+  DestArgs dest;
+};
+
+// gamma alone (roofline.py:68-104), one thread per record; NaN where the
+// reference's assertion 0 <= gamma <= 1 fails.
+__global__ __launch_bounds__(kBlock) void roofline_gamma_kernel(const GammaArgs a) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= a.n) return;
+  const double t = a.run_time_ns[i], eff = a.flop_sp_efficiency[i];
+  const double total_gb = (a.dram_read_bytes[i] + a.dram_write_bytes[i]) * 0x1p-30;
+  const double scaled = div_const<C100>(eff) * a.peak_gflops * t;
+  double num_gflops = div_const<C1e9>(scaled);
+  if (!(div_const_safe(eff) && div_const_safe(scaled)))
+    num_gflops = origin_gflops_exact(a.peak_gflops, eff, t);
+  const double gamma = roofline_gamma(a.dest, num_gflops, total_gb, true);
+  a.out_gamma[i] = (gamma >= 0 && gamma <= 1) ? gamma : __builtin_nan("");
+}
+
 struct RatioArgs {
   const float* pred;          // [(n_dest + 1)][n_ops]; the last row is the origin
   const double* run_time_ms;  // [n_ops]
@@ -287,6 +313,37 @@ int hbt_wave_scale_sum(const hbt_device_table* table, int64_t n, const int32_t* 
     hipLaunchKernelGGL(wave_scale_sum_kernel<true>, grid, dim3(kBlock), 0, stream, a);
   else
     hipLaunchKernelGGL(wave_scale_sum_kernel<false>, grid, dim3(kBlock), 0, stream, a);
+  return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
+}
+
+int hbt_roofline_gamma(const hbt_device_spec* origin, const hbt_device_spec* dest, int64_t n,
+                       const double* run_time_ns, const double* flop_sp_efficiency,
+                       const double* dram_read_bytes, const double* dram_write_bytes,
+                       double* out_gamma, void* hip_stream) {
+  using namespace hbt;
+  if (origin == nullptr || dest == nullptr || n < 0) return HBT_EINVAL;
+  int rc = hbt_device_spec_check(origin);
+  if (rc == HBT_OK) rc = hbt_device_spec_check(dest);
+  if (rc != HBT_OK) return rc;
+  if (n == 0) return HBT_OK;
+  if (!run_time_ns || !flop_sp_efficiency || !dram_read_bytes || !dram_write_bytes || !out_gamma)
+    return HBT_EINVAL;
+  const void* cols[] = {run_time_ns, flop_sp_efficiency, dram_read_bytes, dram_write_bytes,
+                        out_gamma};
+  for (const void* p : cols)
+    if (reinterpret_cast<uintptr_t>(p) % 8 != 0) return HBT_EALIGN;
+  const int64_t blocks = (n + kBlock - 1) / kBlock;
+  if (blocks > 0x7fffffff) return HBT_ESIZE;
+  if (hbt_device_count() <= 0) return HBT_EHIP;
+  GammaArgs a{};
+  a.n = n;
+  a.run_time_ns = run_time_ns; a.flop_sp_efficiency = flop_sp_efficiency;
+  a.dram_read_bytes = dram_read_bytes; a.dram_write_bytes = dram_write_bytes;
+  a.out_gamma = out_gamma;
+  a.peak_gflops = origin->peak_gflops;
+  a.dest = make_dest_args(*origin, *dest);
+  hipLaunchKernelGGL(roofline_gamma_kernel, dim3((unsigned)blocks), dim3(kBlock), 0,
+                     static_cast<hipStream_t>(hip_stream), a);
   return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
 }
 

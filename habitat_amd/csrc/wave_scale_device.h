@@ -186,6 +186,24 @@ __device__ __forceinline__ double log2_count(double log2_lane, int32_t count) {
   return kLog2Int[count & 63];
 }
 
+// roofline.py:78-101 for one record and destination.  With I = gflops / gb the
+// reference takes 0.5 * R / I above the ridge point R and 1 - 0.5 / R * I
+// below; both are formed here from one division by choosing its operands
+// first.  The choice compares gflops with R * gb instead of I with R, which can
+// differ only within an ulp of the ridge, where the two expressions agree
+// (gamma = 1/2).  A record without metrics takes the no-metrics strategy
+// (resimplified.py:25-40): unchanged when small, else t * bw_ratio; with gamma = 1
+// the roofline expressions reduce to exactly that.
+__device__ __forceinline__ double roofline_gamma(const DestArgs& p, double num_gflops,
+                                                 double total_gb, bool metrics) {
+  const bool above = total_gb > 0 && num_gflops > p.ridge * total_gb;
+  const double q = (above ? p.half_ridge * total_gb : num_gflops) /
+                   (above ? num_gflops : total_gb);
+  double gamma = above ? q : p.neg_half_over_ridge * q + 1.;
+  gamma = (total_gb == 0) ? 0. : gamma;
+  return (num_gflops < 1e-9 || !metrics) ? 1. : gamma;
+}
+
 template <bool FAST, bool PERMUTE>
 __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn& r,
                                                const RecordMid& m, double log2_lane) {
@@ -194,20 +212,7 @@ __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn
   o.occ_d = occupancy_dev<FAST>(p.dev, r.block, r.smem_total, m.smem, regs_d);
   o.wave_d = mul_small(p.dev.num_sms, o.occ_d);
 
-  // roofline.py:86-101.  With I = gflops / gb the reference takes
-  // 0.5 * R / I above the ridge point R and 1 - 0.5 / R * I below; both are
-  // formed here from one division by choosing its operands first.  The choice
-  // compares gflops with R * gb instead of I with R, which can differ only
-  // within an ulp of the ridge, where the two expressions agree (gamma = 1/2).
-  const bool above = m.total_gb > 0 && m.num_gflops > p.ridge * m.total_gb;
-  const double q = (above ? p.half_ridge * m.total_gb : m.num_gflops) /
-                   (above ? m.num_gflops : m.total_gb);
-  double gamma = above ? q : p.neg_half_over_ridge * q + 1.;
-  gamma = (m.total_gb == 0) ? 0. : gamma;
-  // A record without metrics takes the no-metrics strategy
-  // (resimplified.py:25-40): unchanged when small, else t * bw_ratio.  With
-  // gamma = 1 the roofline expressions below reduce to exactly that.
-  gamma = (m.num_gflops < 1e-9 || !r.metrics) ? 1. : gamma;
+  const double gamma = roofline_gamma(p, m.num_gflops, m.total_gb, r.metrics);
   const bool bad_gamma = !(gamma >= 0 && gamma <= 1);
 
   // `a // wave_o == 0 and a // wave_d == 0`: the second test, and its division

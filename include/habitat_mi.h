@@ -194,6 +194,18 @@ int hbt_wave_scale_sum(const hbt_device_table *table, int64_t n, const int32_t *
                        double *out_sum, int32_t *out_bad, void *hip_stream);
 
 /*
+ * The roofline exponent alone, _roofline_gamma
+ * (analysis/wave_scaling/roofline.py:68-104) with _ridge_point (:107-108), for n
+ * records that all have their three metrics: out_gamma[n] fp64, NaN where the
+ * reference's assertion 0 <= gamma <= 1 fails.  hbt_wave_scale computes the
+ * same value internally; this entry exists so that it can be inspected.
+ */
+int hbt_roofline_gamma(const hbt_device_spec *origin, const hbt_device_spec *dest, int64_t n,
+                       const double *run_time_ns, const double *flop_sp_efficiency,
+                       const double *dram_read_bytes, const double *dram_write_bytes,
+                       double *out_gamma, void *hip_stream);
+
+/*
  * The last step of the MLP-predicted operations for a device sweep
  * (analysis/predictor.py:132-148 with :182,218,238,283): pred is
  * [(n_dest + 1)][n_ops] fp32 MLP outputs, the last row evaluated with the

@@ -268,6 +268,44 @@ def test_ragged_sizes_single_and_multi_destination(n):
     check(rec, Device.V100, dests, wave_scale(kr, Device.V100, dests))
 
 
+def test_roofline_gamma_alone():
+    """Row a-4 on its own: gamma of every record against the oracle's Python
+    (bit-identical operation order), NaN exactly where the reference asserts."""
+    from habitat_amd.analysis.wave_scaling.batch import roofline_gamma
+    from oracle import wave_scaling as ows
+    rec = adversarial_records(20_000, 23)
+    kr = KernelRecords.from_numpy(rec)
+    for origin, dest in ((Device.V100, Device.MI355X), (Device.T4, Device.P100)):
+        got = roofline_gamma(kr, origin, dest).cpu().numpy()
+        o, d = odev(origin), odev(dest)
+        n_bad = n_mid = 0
+        for i in range(got.shape[0]):
+            row = {k: rec[k][i].item() for k in ("run_time_ns", "flop_sp_efficiency",
+                                                 "dram_read_bytes", "dram_write_bytes")}
+            try:
+                want = ows.gamma(row, o, d)
+            except AssertionError:
+                assert math.isnan(got[i]), (i, row)
+                n_bad += 1
+                continue
+            # abs: where the reference's intensity overflows to infinity (bytes in the
+            # subnormal range) its gamma is exactly 0; the kernel's single division
+            # gives the true quotient, some 1e-315
+            assert got[i] == pytest.approx(want, rel=1e-12, abs=1e-290), (i, row, got[i], want)
+            n_mid += 0 < want < 1
+        assert n_bad > 100 and n_mid > 1000
+    # the scalar face, and the ridge point
+    from habitat_amd.analysis.wave_scaling.roofline import _ridge_point, _roofline_gamma
+    from test_api_gpu import make_kernel
+    row = {k: v[5].item() for k, v in synthetic.kernel_records(8, Device.V100, seed=1)[0].items()}
+    k = make_kernel(Device.V100, t_ns=int(row["run_time_ns"]),
+                    metrics=(row["flop_sp_efficiency"], row["dram_read_bytes"],
+                             row["dram_write_bytes"]))
+    assert _roofline_gamma(k, Device.V100, Device.T4) == pytest.approx(
+        ows.gamma(row, odev(Device.V100), odev(Device.T4)), rel=1e-12)
+    assert _ridge_point(Device.V100) == 6716 / 739
+
+
 def test_wave_counts_are_the_reference_quotients():
     rec = adversarial_records(5000, 17)
     kr = KernelRecords.from_numpy(rec)
