@@ -40,12 +40,13 @@ def __getattr__(name):
 
 
 _SUBMODULES = [
-    "analysis", "analysis.arguments", "analysis.kernels", "analysis.metrics",
+    "analysis", "analysis.arguments", "analysis.device", "analysis.kernels", "analysis.metrics",
     "analysis.operation", "analysis.predictor", "analysis.run_time", "analysis.trace",
     "analysis.mlp", "analysis.mlp.devices", "analysis.mlp.mlp",
     "analysis.wave_scaling", "analysis.wave_scaling.common", "analysis.wave_scaling.metadata",
     "analysis.wave_scaling.resimplified", "analysis.wave_scaling.roofline",
-    "analysis.wave_scaling.unified", "data", "device",
+    "analysis.wave_scaling.unified", "analysis.wave_scaling.batch", "analysis.wave_scaling.cdna",
+    "analysis.report", "analysis.sweep", "data", "device",
 ]
 
 

@@ -208,7 +208,11 @@ def test_habitat_alias_imports():
     from habitat.analysis.kernels import MeasuredKernel, PredictedKernel, KernelInstance
     from habitat.analysis.metrics import Metric  # noqa: F401
     from habitat.analysis.wave_scaling.metadata import NullMetadataManager
+    from habitat.analysis.device import _Device  # noqa: F401
+    from habitat.analysis.wave_scaling.roofline import _ridge_point
+    from habitat.analysis.trace import Trace  # noqa: F401  (no data files needed to import)
     import habitat
+    assert _ridge_point(habitat.Device.T4) == 1804 / 239
     assert habitat.Device.V100.num_sms == 80
     k = KernelInstance("k", 4096, 256, 0, 0, 32, 1000000)
     assert calculate_wave_info(k, habitat.Device.V100, habitat.Device.P100,
