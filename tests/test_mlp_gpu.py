@@ -104,6 +104,19 @@ def test_few_rows_path_and_fused_kernel_agree_on_the_same_rows():
     assert np.array_equal(alone, rp.predict_batch(x[:300]).cpu().numpy())
 
 
+@pytest.mark.parametrize("hidden", [0, 1, 3])
+@pytest.mark.parametrize("rows", [5, 130, 600])
+def test_other_depths(hidden, rows):
+    """Networks with no, one and three hidden layers through both paths (the
+    kernels take the depth from the handle; without hidden layers the final dot
+    product reads fc1's single partial)."""
+    rp = make("lstm", seed=4, hidden=hidden)
+    x, mu, sigma = synthetic.mlp_features("lstm", rows, seed=8)
+    rp.set_normalization(mu, sigma)
+    y = rp.predict_batch(x).cpu().numpy()
+    assert_close(y, omlp.forward_fp64(rp.model.state_dict(), x, mu, sigma))
+
+
 def test_empty_batch():
     rp = make("bmm")
     rp.set_normalization(np.zeros(8), np.ones(8))
