@@ -117,6 +117,38 @@ def test_other_depths(hidden, rows):
     assert_close(y, omlp.forward_fp64(rp.model.state_dict(), x, mu, sigma))
 
 
+@pytest.mark.parametrize("features", [21, 36, 60])
+def test_wide_inputs_up_to_64_features(features):
+    """The C ABI takes up to 64 input features (fc1's K padded to 32 or 64);
+    the reference's predictors stop at 12, so this goes through a model class of
+    the test's own."""
+    from habitat_amd.analysis.mlp.mlp import _DeviceMLP, _OperationMLP
+
+    Wide = type("Wide", (_OperationMLP,), {"features": ["f%d" % i for i in range(features)]})
+
+    torch.manual_seed(9)
+    model = Wide(1, 1024)
+    rng = np.random.default_rng(9)
+    f = features + 4
+    x = rng.normal(3.0, 2.0, size=(700, f))
+    mu, sigma = x.mean(axis=0), x.std(axis=0)
+    gpu = _DeviceMLP(model, mu, sigma)
+    want = omlp.forward_fp64(model.state_dict(), x, mu, sigma)
+    for rows in (50, 700):
+        y = gpu.forward(torch.from_numpy(x[:rows]).cuda()).cpu().numpy()
+        # outputs of this random two-layer net are sums of O(1) terms that nearly
+        # cancel: the floor of the relative tolerance is the terms' magnitude
+        assert_close(y, want[:rows], floor=1.0)
+        y32 = omlp.forward_fp32(model.state_dict(), x[:rows], mu, sigma)
+        assert np.max(np.abs(y - want[:rows])) <= 4 * np.max(np.abs(y32 - want[:rows])) + 1e-7
+    # 65 features do not fit
+    TooWide = type("TooWide", (_OperationMLP,), {"features": ["f%d" % i for i in range(61)]})
+    from habitat_amd import _lib
+    with pytest.raises(_lib.HabitatLibraryError) as e:
+        _DeviceMLP(TooWide(1, 1024), np.zeros(65), np.ones(65))
+    assert e.value.code == _lib.HBT_ESIZE
+
+
 def test_empty_batch():
     rp = make("bmm")
     rp.set_normalization(np.zeros(8), np.ones(8))
