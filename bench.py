@@ -301,7 +301,7 @@ def main():
         d = olib.make_device(**dest.as_dict())
         olib.wave_scale(o, d, rec)
         reps, t0 = 0, time.perf_counter()
-        while reps < 3 or (time.perf_counter() - t0 < 5.0 and reps < 100):
+        while reps < 3 or (time.perf_counter() - t0 < 10.0 and reps < 400):
             olib.wave_scale(o, d, rec)
             reps += 1
         c_rate = reps * args.records / (time.perf_counter() - t0)
