@@ -17,6 +17,7 @@ _TABLE = {
     # this build's synthetic destination
     "MI355X":    dict(mem=288, mem_type="HBM3E", mem_bw=8000, num_sm=256, double=78.6, single=157.3,  half=2500.0),
 }
+_TABLE["MI355X_cdna"] = _TABLE["MI355X"]   # the same GPU under its compute-unit description
 
 DEVICE_PARAMS = ["mem", "mem_bw", "num_sm", "single"]
 
