@@ -122,6 +122,85 @@ def tile_records(rec, n):
     return {k: np.tile(v, reps)[:n] for k, v in rec.items()}
 
 
+def mlp_bench(args):
+    """configs[2] (and the other kinds of configs[3], one step each): the fused
+    MLP at full size, the few-rows path, and a torch CPU baseline."""
+    import torch
+    from habitat_amd import synthetic
+    from habitat_amd.analysis.mlp.mlp import RuntimePredictor
+    kind = args.mlp_kind
+    torch.manual_seed(0)
+    rp = RuntimePredictor(kind, 8, 1024)
+    x, mu, sigma = synthetic.mlp_features(kind, args.mlp_rows, seed=2)
+    rp.set_normalization(mu, sigma)
+    xg = torch.from_numpy(x).cuda()
+    yg = torch.empty(args.mlp_rows, dtype=torch.float32, device="cuda")
+    f_in = x.shape[1]
+    flops_per_row = 2.0 * (f_in * 1024 + 8 * 1024 * 1024 + 1024)
+    mlp_call = lambda: rp.predict_batch(xg, out=yg)
+    m_wall, m_launch = time_steps(mlp_call, args.mlp_steps, 1)
+    tflops = flops_per_row * args.mlp_rows / (m_launch * 1e-3) / 1e12
+    mlp = {"metric": "MLP op-predictions/s", "value": args.mlp_rows / (m_wall * 1e-3),
+           "unit": "rows/s", "steps": args.mlp_steps, "ms_per_step": m_wall, "dtype": "f32",
+           "config": {"workload": "configs[2]: %s MLP, %d rows x %d raw fp64 features, "
+                                  "fc1 + 8 x 1024 hidden + fc2, seed-0 random init"
+                                  % (kind, args.mlp_rows, f_in)},
+           "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_FP32_PEAK_TFLOPS,
+                        "unit": "TFLOP/s", "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
+                        "traffic": (MLP_TRAFFIC_BYTES_PER_ROW * args.mlp_rows
+                                    if kind == "conv2d" else None),
+                        "kernel": "mlp_fused_kernel<4>",
+                        "launch_ms": m_launch, "flops_per_row": flops_per_row}}
+    if not args.no_cpu:
+        from oracle import mlp as omlp
+        sd = rp.model.state_dict()
+        m = min(32768, args.mlp_rows)
+        threads = torch.get_num_threads()
+        omlp.forward_fp32(sd, x[:1024], mu, sigma)
+        t0 = time.perf_counter()
+        omlp.forward_fp32(sd, x[:m], mu, sigma)
+        dt = time.perf_counter() - t0
+        mlp["cpu_baseline"] = {
+            "value": m / dt, "unit": "rows/s", "cores": threads, "kind": "port",
+            "sample": "oracle/mlp.py forward_fp32 (torch CPU fp32, one batched forward) on "
+                      "the first %d rows, %d torch threads" % (m, threads)}
+    # few rows: the reference's own call pattern is one row per call (mlp.py:252-267)
+    few = {}
+    for rows in (1, 108, 512):
+        xs = xg[:rows].contiguous()
+        ys = torch.empty(rows, dtype=torch.float32, device="cuda")
+        _, f_launch = time_steps(lambda: rp.predict_batch(xs, out=ys), 50, 5)
+        few["rows_%d_us" % rows] = f_launch * 1e3
+    if not args.no_cpu:
+        from oracle import mlp as omlp
+        sd = rp.model.state_dict()
+        omlp.forward_fp32(sd, x[:1], mu, sigma)
+        t0 = time.perf_counter()
+        for i in range(20):
+            omlp.forward_fp32(sd, x[i:i + 1], mu, sigma)
+        few["cpu_rows_1_us"] = (time.perf_counter() - t0) / 20 * 1e6
+    few["note"] = ("up to 512 rows: one launch per layer over the whole GPU (mlp_layer_kernel); "
+                   "cpu_rows_1_us: torch CPU fp32, batch 1, as the reference predicts")
+    mlp["few_rows"] = few
+    others = {}
+    for other in [k for k in args.mlp_other_kinds.split(",") if k and k != kind]:
+        torch.manual_seed(0)
+        rpo = RuntimePredictor(other, 8, 1024)
+        xo, muo, sgo = synthetic.mlp_features(other, args.mlp_rows, seed=2)
+        rpo.set_normalization(muo, sgo)
+        xog = torch.from_numpy(xo).cuda()
+        _, o_launch = time_steps(lambda: rpo.predict_batch(xog, out=yg), 1, 1)
+        fl = 2.0 * (xo.shape[1] * 1024 + 8 * 1024 * 1024 + 1024)
+        tf = fl * args.mlp_rows / (o_launch * 1e-3) / 1e12
+        others[other] = {"rows": args.mlp_rows, "launch_ms": o_launch,
+                         "value": args.mlp_rows / (o_launch * 1e-3), "unit": "rows/s",
+                         "achieved": tf, "frac": tf / MFMA_FP32_PEAK_TFLOPS}
+        del rpo, xog
+    if others:
+        mlp["other_kinds"] = others
+    return mlp
+
+
 def sweep_bench(args, origin):
     """configs[4]: predicted iteration time of one trace on D devices."""
     import numpy as np
@@ -248,7 +327,6 @@ def main():
     import numpy as np
     import torch
     from habitat_amd import Device, synthetic
-    from habitat_amd.analysis.mlp.mlp import RuntimePredictor
     from habitat_amd.analysis.wave_scaling.batch import KernelRecords, WaveScaleOutput
 
     if not torch.cuda.is_available():
@@ -293,8 +371,18 @@ def main():
                      "bytes_per_record": BYTES_PER_RECORD},
     }
 
+    def attempt(key, section):
+        """A secondary section must not cost the headline line: on failure its
+        entry says what went wrong."""
+        try:
+            value = section()
+        except Exception as exc:   # noqa: BLE001 - reported, not swallowed
+            value = {"error": "%s: %s" % (type(exc).__name__, exc)}
+        if value is not None:
+            result[key] = value
+
     # ---------------- CPU baseline on the same records ----------------
-    if not args.no_cpu:
+    def cpu_section():
         from oracle import lib as olib
         from oracle import wave_scaling as ows
         o = olib.make_device(**origin.as_dict())
@@ -311,7 +399,7 @@ def main():
         for row in rows:
             ows.unified(row, o, d)
         py_rate = m / (time.perf_counter() - t0)
-        result["cpu_baseline"] = {
+        return {
             "value": c_rate, "unit": "records/s", "cores": 1, "kind": "port",
             "sample": "oracle/wave_scaling.c (per-record C restatement of the reference's "
                       "Python, libm pow) over the same %d records x %d passes, one thread of %d "
@@ -321,110 +409,47 @@ def main():
                 "sample": "oracle/wave_scaling.py, one Python call chain per record as the "
                           "reference does, first %d records" % m}}
 
+    if not args.no_cpu:
+        attempt("cpu_baseline", cpu_section)
+
     # ---------------- the same kernel beyond the last-level cache ----------------
-    if not args.no_large and args.large_records > args.records:
-        del call, records, out
+    def large_section():
         big = KernelRecords.from_numpy(tile_records(rec, args.large_records))
         big_out = WaveScaleOutput(big.n, 1, big.device, waves=False, status=True)
         big_call = WaveScaleCall(big, origin, dest, big_out)
         steps = max(5, min(args.steps, 40))
         b_wall, b_launch = time_steps(big_call, steps, min(args.warmup, 20))
         b_ach = BYTES_PER_RECORD * big.n / (b_launch * 1e-3) / 1e9
-        result["large"] = {"records": big.n, "steps": steps, "ms_per_step": b_wall,
-                           "value": big.n / (b_wall * 1e-3), "unit": "records/s",
-                           "roofline": {"bound": "hbm", "achieved": b_ach, "peak": HBM_PEAK_GBS,
-                                        "unit": "GB/s", "frac": b_ach / HBM_PEAK_GBS,
-                                        "launch_us": b_launch * 1e3}}
-        del big_call, big, big_out
+        return {"records": big.n, "steps": steps, "ms_per_step": b_wall,
+                "value": big.n / (b_wall * 1e-3), "unit": "records/s",
+                "roofline": {"bound": "hbm", "achieved": b_ach, "peak": HBM_PEAK_GBS,
+                             "unit": "GB/s", "frac": b_ach / HBM_PEAK_GBS,
+                             "launch_us": b_launch * 1e3}}
+
+    del call, records, out
+    if not args.no_large and args.large_records > args.records:
+        attempt("large", large_section)
         torch.cuda.empty_cache()
 
     # ---------------- MLP, configs[2] ----------------
     if not args.no_mlp:
-        kind = args.mlp_kind
-        torch.manual_seed(0)
-        rp = RuntimePredictor(kind, 8, 1024)
-        x, mu, sigma = synthetic.mlp_features(kind, args.mlp_rows, seed=2)
-        rp.set_normalization(mu, sigma)
-        xg = torch.from_numpy(x).cuda()
-        yg = torch.empty(args.mlp_rows, dtype=torch.float32, device="cuda")
-        f_in = x.shape[1]
-        flops_per_row = 2.0 * (f_in * 1024 + 8 * 1024 * 1024 + 1024)
-        mlp_call = lambda: rp.predict_batch(xg, out=yg)
-        m_wall, m_launch = time_steps(mlp_call, args.mlp_steps, 1)
-        tflops = flops_per_row * args.mlp_rows / (m_launch * 1e-3) / 1e12
-        mlp = {"metric": "MLP op-predictions/s", "value": args.mlp_rows / (m_wall * 1e-3),
-               "unit": "rows/s", "steps": args.mlp_steps, "ms_per_step": m_wall, "dtype": "f32",
-               "config": {"workload": "configs[2]: %s MLP, %d rows x %d raw fp64 features, "
-                                      "fc1 + 8 x 1024 hidden + fc2, seed-0 random init"
-                                      % (kind, args.mlp_rows, f_in)},
-               "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_FP32_PEAK_TFLOPS,
-                            "unit": "TFLOP/s", "frac": tflops / MFMA_FP32_PEAK_TFLOPS,
-                            "traffic": (MLP_TRAFFIC_BYTES_PER_ROW * args.mlp_rows
-                                        if kind == "conv2d" else None),
-                            "kernel": "mlp_fused_kernel<4>",
-                            "launch_ms": m_launch, "flops_per_row": flops_per_row}}
-        if not args.no_cpu:
-            from oracle import mlp as omlp
-            sd = rp.model.state_dict()
-            m = min(32768, args.mlp_rows)
-            threads = torch.get_num_threads()
-            omlp.forward_fp32(sd, x[:1024], mu, sigma)
-            t0 = time.perf_counter()
-            omlp.forward_fp32(sd, x[:m], mu, sigma)
-            dt = time.perf_counter() - t0
-            mlp["cpu_baseline"] = {
-                "value": m / dt, "unit": "rows/s", "cores": threads, "kind": "port",
-                "sample": "oracle/mlp.py forward_fp32 (torch CPU fp32, one batched forward) on "
-                          "the first %d rows, %d torch threads" % (m, threads)}
-        # few rows: the reference's own call pattern is one row per call (mlp.py:252-267)
-        few = {}
-        for rows in (1, 108, 512):
-            xs = xg[:rows].contiguous()
-            ys = torch.empty(rows, dtype=torch.float32, device="cuda")
-            _, f_launch = time_steps(lambda: rp.predict_batch(xs, out=ys), 50, 5)
-            few["rows_%d_us" % rows] = f_launch * 1e3
-        if not args.no_cpu:
-            from oracle import mlp as omlp
-            sd = rp.model.state_dict()
-            omlp.forward_fp32(sd, x[:1], mu, sigma)
-            t0 = time.perf_counter()
-            for i in range(20):
-                omlp.forward_fp32(sd, x[i:i + 1], mu, sigma)
-            few["cpu_rows_1_us"] = (time.perf_counter() - t0) / 20 * 1e6
-        few["note"] = ("up to 512 rows: one launch per layer over the whole GPU (mlp_layer_kernel); "
-                       "cpu_rows_1_us: torch CPU fp32, batch 1, as the reference predicts")
-        mlp["few_rows"] = few
-        others = {}
-        for other in [k for k in args.mlp_other_kinds.split(",") if k and k != kind]:
-            torch.manual_seed(0)
-            rpo = RuntimePredictor(other, 8, 1024)
-            xo, muo, sgo = synthetic.mlp_features(other, args.mlp_rows, seed=2)
-            rpo.set_normalization(muo, sgo)
-            xog = torch.from_numpy(xo).cuda()
-            _, o_launch = time_steps(lambda: rpo.predict_batch(xog, out=yg), 1, 1)
-            fl = 2.0 * (xo.shape[1] * 1024 + 8 * 1024 * 1024 + 1024)
-            tf = fl * args.mlp_rows / (o_launch * 1e-3) / 1e12
-            others[other] = {"rows": args.mlp_rows, "launch_ms": o_launch,
-                             "value": args.mlp_rows / (o_launch * 1e-3), "unit": "rows/s",
-                             "achieved": tf, "frac": tf / MFMA_FP32_PEAK_TFLOPS}
-            del rpo, xog
-        if others:
-            mlp["other_kinds"] = others
-        result["mlp"] = mlp
+        attempt("mlp", lambda: mlp_bench(args))
 
     # ---------------- configs[4]: one trace, a sweep of destination devices ----------------
     if not args.no_sweep:
-        result["sweep"] = sweep_bench(args, origin)
+        attempt("sweep", lambda: sweep_bench(args, origin))
 
     # ---------------- what this box itself can do (ceilings under the published peaks) ----------
-    if not args.no_ceilings:
+    def ceilings_section():
         from habitat_amd import device_info
         name, _ = device_info.local_device(0)
         m = device_info.measure()
-        result["measured_ceilings"] = {
-            "device": name, "copy_GBps_read_plus_write": m["copy_gbps"],
-            "fp32_mfma_TFLOPs": m["fp32_mfma_gflops"] / 1e3,
-            "fp32_vector_fma_TFLOPs": m["fp32_fma_gflops"] / 1e3}
+        return {"device": name, "copy_GBps_read_plus_write": m["copy_gbps"],
+                "fp32_mfma_TFLOPs": m["fp32_mfma_gflops"] / 1e3,
+                "fp32_vector_fma_TFLOPs": m["fp32_fma_gflops"] / 1e3}
+
+    if not args.no_ceilings:
+        attempt("measured_ceilings", ceilings_section)
 
     print(json.dumps(result))
 
