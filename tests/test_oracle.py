@@ -247,3 +247,68 @@ def test_predictor_arithmetic():
     assert opred.trace_ms([fwd + bwd, 1.6, 0.0]) == pytest.approx(6.1)
     # a pass without kernels keeps its measured time
     assert opred.wave_scaled_pass_ms(0.7, [], []) == pytest.approx(0.7)
+
+
+def random_device_specs(count, seed):
+    """Device descriptions far from the shipped ones: every compute capability
+    the routine distinguishes, odd warp sizes, limits from tiny to huge,
+    occasional zeros and negatives."""
+    rng = np.random.default_rng(seed)
+    pick = lambda values: int(rng.choice(values))
+    specs = []
+    for _ in range(count):
+        warp = pick([32, 32, 32, 64, 64, 16, 24, 48, 96, 128, 1, 1000])
+        threads_block = pick([1024, 1024, 512, 2048, 1536, 100, 0, 65536])
+        specs.append(dict(
+            compute_major=pick([3, 5, 6, 6, 7, 7, 7, 8, 2, 9, 0]),
+            compute_minor=pick([0, 0, 1, 2, 5, 7]),
+            max_threads_per_block=threads_block,
+            max_threads_per_multiprocessor=pick([2048, 1024, 1536, 4096, 768, 64, 0, 1 << 20]),
+            regs_per_block=pick([65536, 32768, 131072, 65536, 4096, 0, 1 << 22, 100000]),
+            regs_per_multiprocessor=pick([65536, 131072, 262144, 32768, 100000, 0, 1 << 22]),
+            warp_size=warp,
+            shared_mem_per_block=pick([49152, 65536, 98304, 16384, 163840, 1000, 0, 1 << 21]),
+            shared_mem_per_multiprocessor=pick([65536, 98304, 102400, 163840, 49152, 32768, 8192,
+                                                100, 0, 1 << 21]),
+            num_sms=pick([1, 14, 80, 256, 1000]),
+            shared_mem_per_block_optin=pick([0, 49152, 98304]),
+            mem_bandwidth_gb=900, base_clock_mhz=1300, peak_gflops_per_second=14000))
+    return specs
+
+
+def test_random_device_specs_against_the_compiled_reference():
+    """The oracle, the library's host routine and its 32-bit kernel model on 300
+    random device descriptions x 400 launches (ordinary and out-of-range),
+    against the reference's own routine compiled in place."""
+    if olib.ref() is None:
+        pytest.skip("oracle/_ref was not built (reference tree not mounted)")
+    import ctypes
+    from habitat_amd import DeviceProperties, _lib
+    rng = np.random.default_rng(5)
+    n = 400
+    odd = np.array([0, -1, 1, 31, 33, 255, 256, 257, 1023, 1025, 65535, 65536, 65537, 1 << 20,
+                    (1 << 31) - 1, -(1 << 31), -256, -510, -511])
+    mix = lambda ordinary: np.where(rng.random(n) < 0.8, ordinary, rng.choice(odd, n)).astype(np.int32)
+    accepted = model32_checked = 0
+    for props in random_device_specs(300, 17):
+        block = mix(rng.integers(1, 2100, n))
+        dyn = mix(rng.integers(0, 120000, n))
+        stat = mix(rng.integers(0, 60000, n))
+        regs = mix(rng.integers(0, 300, n))
+        d = oracle_device(props)
+        want = olib.ref_occupancy_batch(d, block, dyn, stat, regs)
+        assert np.array_equal(olib.occupancy_batch(d, block, dyn, stat, regs), want), props
+        accepted += bool(want.any())
+        dev = DeviceProperties(name="r", **props)
+        for fn in ("hbt_occupancy_host_batch", "hbt_occupancy_host_model32_batch"):
+            out = np.full(n, -9, np.int32)
+            rc = getattr(_lib.lib(), fn)(
+                ctypes.byref(dev.spec), n, *[a.ctypes.data_as(ctypes.c_void_p)
+                                             for a in (block, dyn, stat, regs)],
+                out.ctypes.data_as(ctypes.c_void_p))
+            if fn.endswith("model32_batch") and rc == _lib.HBT_ESPEC:
+                continue          # a limit of 2^20 or more: the kernel uses the 64-bit model
+            assert rc == 0, (fn, rc, props)
+            assert np.array_equal(out, want), (fn, props)
+            model32_checked += fn.endswith("model32_batch")
+    assert accepted > 60 and model32_checked > 150
