@@ -280,7 +280,8 @@ int hbt_wave_scale_sum(const hbt_device_table* table, int64_t n, const int32_t* 
                 !run_time_ns || !flop_sp_efficiency || !dram_read_bytes || !dram_write_bytes))
     return HBT_EINVAL;
   const int64_t blocks = (n + kBlock - 1) / kBlock;
-  if (blocks > 0x7fffffff || (int64_t)n_segments * table->n_dest > ((int64_t)1 << 40))
+  // (the clearing launch covers n_dest * n_segments sums with 256 threads per block)
+  if (blocks > 0x7fffffff || (int64_t)n_segments * table->n_dest > ((int64_t)1 << 38))
     return HBT_ESIZE;
   int device = -1;
   if (hipGetDevice(&device) != hipSuccess) {
