@@ -444,9 +444,20 @@ def main():
         from habitat_amd import device_info
         name, _ = device_info.local_device(0)
         m = device_info.measure()
-        return {"device": name, "copy_GBps_read_plus_write": m["copy_gbps"],
-                "fp32_mfma_TFLOPs": m["fp32_mfma_gflops"] / 1e3,
-                "fp32_vector_fma_TFLOPs": m["fp32_fma_gflops"] / 1e3}
+        out = {"device": name, "copy_GBps_read_plus_write": m["copy_gbps"],
+               "fp32_mfma_TFLOPs": m["fp32_mfma_gflops"] / 1e3,
+               "fp32_vector_fma_TFLOPs": m["fp32_fma_gflops"] / 1e3}
+        # yardstick for the MLP: the vendor library's fp32 GEMM (+ bias) on one hidden
+        # layer's shape, activations through HBM
+        torch.backends.cuda.matmul.allow_tf32 = False
+        rows = 262144
+        a = torch.randn(rows, 1024, device="cuda")
+        w = torch.randn(1024, 1024, device="cuda")
+        b = torch.randn(1024, device="cuda")
+        y = torch.empty(rows, 1024, device="cuda")
+        _, g_ms = time_steps(lambda: torch.addmm(b, a, w.t(), out=y), 10, 3)
+        out["vendor_fp32_gemm_one_layer_TFLOPs"] = 2.0 * rows * 1024 * 1024 / (g_ms * 1e-3) / 1e12
+        return out
 
     if not args.no_ceilings:
         attempt("measured_ceilings", ceilings_section)
