@@ -447,6 +447,11 @@ def main():
         out = {"device": name, "copy_GBps_read_plus_write": m["copy_gbps"],
                "fp32_mfma_TFLOPs": m["fp32_mfma_gflops"] / 1e3,
                "fp32_vector_fma_TFLOPs": m["fp32_fma_gflops"] / 1e3}
+        # yardstick for wave scaling: its loads and stores without the arithmetic
+        out["record_stream_GBps_at_%d_records" % args.records] = device_info.record_stream_gbps(
+            args.records, args.warmup, args.steps)
+        out["record_stream_GBps_at_%d_records" % args.large_records] = (
+            device_info.record_stream_gbps(args.large_records, 20, 40))
         # yardstick for the MLP: the vendor library's fp32 GEMM (+ bias) on one hidden
         # layer's shape, activations through HBM
         torch.backends.cuda.matmul.allow_tf32 = False

@@ -53,6 +53,16 @@ def measure(iters=20000, copy_bytes=1 << 30):
     return out
 
 
+def record_stream_gbps(records, warmup=2000, launches=2000):
+    """GB/s (68 bytes per record) of a kernel doing only the loads and stores of
+    wave scaling on `records` records: the data-movement ceiling at that size."""
+    v = ctypes.c_double(0)
+    _lib.check(_lib.lib().hbt_measure_record_stream_gbps(records, warmup, launches,
+                                                         ctypes.byref(v)),
+               "hbt_measure_record_stream_gbps")
+    return v.value
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--device", type=int, default=0)

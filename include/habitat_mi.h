@@ -266,12 +266,18 @@ void hbt_mlp_destroy(hbt_mlp *mlp);
  * role of the reference's flop_test kernel (cpp/src/cuda/diagnostics.cu:9-25,
  * tools/device-metadata/measure_peak_flops.py:10-18); hbt_measure_fp32_mfma_gflops
  * does the same with v_mfma_f32_32x32x2_f32; hbt_measure_copy_gbps times a
- * device-to-device copy of `bytes` (read + write counted).
+ * device-to-device copy of `bytes` (read + write counted);
+ * hbt_measure_record_stream_gbps times a kernel that performs the loads and
+ * stores of hbt_wave_scale on n records (same columns, same access pattern) and
+ * no arithmetic, `launches` times after `warmup` untimed ones, and reports
+ * 68 bytes per record over the launch time: the data-movement ceiling the
+ * wave-scaling kernel can be held against at that size.
  */
 int hbt_local_device_spec(int device, hbt_device_spec *out, char *name, size_t name_len);
 int hbt_measure_fp32_fma_gflops(int iters, double *out_gflops);
 int hbt_measure_fp32_mfma_gflops(int iters, double *out_gflops);
 int hbt_measure_copy_gbps(size_t bytes, double *out_gbps);
+int hbt_measure_record_stream_gbps(int64_t n, int warmup, int launches, double *out_gbps);
 
 #ifdef __cplusplus
 }
