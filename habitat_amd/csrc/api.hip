@@ -146,7 +146,7 @@ int hbt_wave_scale(const hbt_device_spec* origin, const hbt_device_spec* dests, 
   if (!num_blocks || !block_size || !dynamic_smem || !static_smem || !regs || !run_time_ns ||
       !flop_sp_efficiency || !dram_read_bytes || !dram_write_bytes || !out_time_ns)
     return HBT_EINVAL;
-  if (n > ((int64_t)1 << 40)) return HBT_ESIZE;
+  if (n > ((int64_t)1 << 36)) return HBT_ESIZE;  // one wavefront per workgroup: the grid stays below 2^31
 
   const void* i32_cols[] = {num_blocks, block_size, dynamic_smem, static_smem, regs, dest_regs,
                             out_occ_origin, out_occ_dest, out_wave_origin, out_wave_dest};

@@ -77,11 +77,11 @@ struct StreamArgs {
 };
 
 // The data movement of the wave-scaling kernel and nothing else: the same nine
-// input and four output columns, two records per thread, 512-thread workgroups,
+// input and four output columns, two records per thread, one wavefront per workgroup,
 // non-temporal accesses; the arithmetic is a few additions so that no load can
 // be dropped.
-__global__ __launch_bounds__(512) void record_stream_kernel(const StreamArgs a) {
-  const uint32_t i = (blockIdx.x * 512u + threadIdx.x) * 2u;
+__global__ __launch_bounds__(64) void record_stream_kernel(const StreamArgs a) {
+  const uint32_t i = (blockIdx.x * 64u + threadIdx.x) * 2u;
   if (i + 2 > a.n) return;
   int32_t s0 = 0, s1 = 0;
   double d0 = 0, d1 = 0;
@@ -284,17 +284,17 @@ int hbt_measure_record_stream_gbps(int64_t n, int warmup, int launches, double* 
   a.out_occ[1] = reinterpret_cast<int32_t*>(p); p += col4;
   a.out_status = reinterpret_cast<uint8_t*>(p);
   a.n = (uint32_t)n;
-  const unsigned blocks = (unsigned)((n / 2 + 511) / 512);
+  const unsigned blocks = (unsigned)((n / 2 + 63) / 64);
   Timer t;
   int rc = t.ok ? HBT_OK : HBT_EHIP;
   float ms = 0.f;
   if (rc == HBT_OK && hipMemsetAsync(base, 0, total, nullptr) != hipSuccess) rc = HBT_EHIP;
   if (rc == HBT_OK) {
     for (int i = 0; i < warmup; ++i)
-      hipLaunchKernelGGL(record_stream_kernel, dim3(blocks), dim3(512), 0, nullptr, a);
+      hipLaunchKernelGGL(record_stream_kernel, dim3(blocks), dim3(64), 0, nullptr, a);
     (void)hipEventRecord(t.e0, nullptr);
     for (int i = 0; i < launches; ++i)
-      hipLaunchKernelGGL(record_stream_kernel, dim3(blocks), dim3(512), 0, nullptr, a);
+      hipLaunchKernelGGL(record_stream_kernel, dim3(blocks), dim3(64), 0, nullptr, a);
     (void)hipEventRecord(t.e1, nullptr);
     if (hipEventSynchronize(t.e1) != hipSuccess ||
         hipEventElapsedTime(&ms, t.e0, t.e1) != hipSuccess || hipGetLastError() != hipSuccess)
