@@ -44,9 +44,9 @@ MLP_TRAFFIC_BYTES_PER_ROW = 33040.0  # profiles/mlp_fused_kernel_conv2d_1M_rows.
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # Defaults long enough to report the sustained rate: for the first ~10 ms
-    # after idle the GPU runs this kernel about 8 % faster than it then settles
-    # to (try --warmup 20 --steps 200).
+    # Defaults long enough to report the rate under continuous launches (some
+    # kernel configurations run several per cent faster for the first
+    # milliseconds after idle).
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=2000)
     ap.add_argument("--records", type=int, default=1_000_000)
