@@ -36,8 +36,8 @@ MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 BYTES_PER_RECORD = 68          # 5 x i32 + 4 x f64 read, f64 + 2 x i32 written
 # Measured L2<->fabric bytes per record (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled
 # on a copy kernel of known size; profiles/wave_scale_kernel_1M_and_64M_records.md):
-# 52.18 read + 17.00 written (the status byte is the 69th).
-TRAFFIC_BYTES_PER_RECORD = 69.18
+# 52.07 read + 17.13 written (the status byte is the 69th).
+TRAFFIC_BYTES_PER_RECORD = 69.20
 MLP_TRAFFIC_BYTES_PER_ROW = 33040.0  # profiles/mlp_fused_kernel_conv2d_1M_rows.md: weights re-streamed per round
 
 
@@ -367,7 +367,7 @@ def main():
                      "traffic": TRAFFIC_BYTES_PER_RECORD * args.records,
                      "traffic_unit": "bytes/launch (FETCH_SIZE + WRITE_SIZE, rocprofv3, "
                                      "copy-calibrated; see profiles/)",
-                     "kernel": "wave_scale_kernel<2, true, true, unsigned int>", "launch_us": launch_ms * 1e3,
+                     "kernel": "wave_scale_kernel<1, true, true, unsigned int>", "launch_us": launch_ms * 1e3,
                      "bytes_per_record": BYTES_PER_RECORD},
     }
 

@@ -146,15 +146,16 @@ int hbt_wave_scale(const hbt_device_spec* origin, const hbt_device_spec* dests, 
   if (!num_blocks || !block_size || !dynamic_smem || !static_smem || !regs || !run_time_ns ||
       !flop_sp_efficiency || !dram_read_bytes || !dram_write_bytes || !out_time_ns)
     return HBT_EINVAL;
-  if (n > ((int64_t)1 << 36)) return HBT_ESIZE;  // one wavefront per workgroup: the grid stays below 2^31
+  if (n > ((int64_t)1 << 36)) return HBT_ESIZE;  // 128 records per workgroup: the grid stays far below 2^31
 
   const void* i32_cols[] = {num_blocks, block_size, dynamic_smem, static_smem, regs, dest_regs,
                             out_occ_origin, out_occ_dest, out_wave_origin, out_wave_dest};
   const void* f64_cols[] = {run_time_ns, flop_sp_efficiency, dram_read_bytes, dram_write_bytes,
                             out_time_ns};
-  // The vectorised kernel accesses kVectorRecords elements at a time: every
+  // The main instantiation accesses kVectorRecords elements at a time: every
   // column, and every destination's row of an output ([n_dest][n]), must be
-  // aligned to that many elements.
+  // aligned to that many elements (with one record per thread that is the
+  // element alignment already required).
   bool vec = true;
   for (const void* p : i32_cols) {
     if (!aligned(p, 4)) return HBT_EALIGN;

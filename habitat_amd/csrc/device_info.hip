@@ -63,10 +63,6 @@ __global__ __launch_bounds__(256) void mfma_peak_kernel(float* out, int iters, f
   out[blockIdx.x * 256 + threadIdx.x] = s;
 }
 
-using i32x2 = int32_t __attribute__((ext_vector_type(2)));
-using f64x2 = double __attribute__((ext_vector_type(2)));
-using u8x2 = uint8_t __attribute__((ext_vector_type(2)));
-
 struct StreamArgs {
   const int32_t* ints[5];
   const double* dbls[4];
@@ -77,36 +73,22 @@ struct StreamArgs {
 };
 
 // The data movement of the wave-scaling kernel and nothing else: the same nine
-// input and four output columns, two records per thread, one wavefront per workgroup,
+// input and four output columns, one record per thread, 128-thread workgroups,
 // non-temporal accesses; the arithmetic is a few additions so that no load can
 // be dropped.
-__global__ __launch_bounds__(64) void record_stream_kernel(const StreamArgs a) {
-  const uint32_t i = (blockIdx.x * 64u + threadIdx.x) * 2u;
-  if (i + 2 > a.n) return;
-  int32_t s0 = 0, s1 = 0;
-  double d0 = 0, d1 = 0;
+__global__ __launch_bounds__(128) void record_stream_kernel(const StreamArgs a) {
+  const uint32_t i = blockIdx.x * 128u + threadIdx.x;
+  if (i >= a.n) return;
+  int32_t s = 0;
+  double d = 0;
 #pragma unroll
-  for (int k = 0; k < 5; ++k) {
-    const i32x2 v = __builtin_nontemporal_load(reinterpret_cast<const i32x2*>(
-        reinterpret_cast<const char*>(a.ints[k]) + (size_t)(i * 4u)));
-    s0 += v[0]; s1 += v[1];
-  }
+  for (int k = 0; k < 5; ++k) s += __builtin_nontemporal_load(a.ints[k] + i);
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const f64x2 v = __builtin_nontemporal_load(reinterpret_cast<const f64x2*>(
-        reinterpret_cast<const char*>(a.dbls[k]) + (size_t)(i * 8u)));
-    d0 += v[0]; d1 += v[1];
-  }
-  const f64x2 t = {d0, d1};
-  __builtin_nontemporal_store(t, reinterpret_cast<f64x2*>(
-      reinterpret_cast<char*>(a.out_time) + (size_t)(i * 8u)));
-  const i32x2 q0 = {s0, s1}, q1 = {s1, s0};
-  __builtin_nontemporal_store(q0, reinterpret_cast<i32x2*>(
-      reinterpret_cast<char*>(a.out_occ[0]) + (size_t)(i * 4u)));
-  __builtin_nontemporal_store(q1, reinterpret_cast<i32x2*>(
-      reinterpret_cast<char*>(a.out_occ[1]) + (size_t)(i * 4u)));
-  const u8x2 st = {(uint8_t)s0, (uint8_t)s1};
-  __builtin_nontemporal_store(st, reinterpret_cast<u8x2*>(a.out_status + (size_t)i));
+  for (int k = 0; k < 4; ++k) d += __builtin_nontemporal_load(a.dbls[k] + i);
+  __builtin_nontemporal_store(d, a.out_time + i);
+  __builtin_nontemporal_store(s, a.out_occ[0] + i);
+  __builtin_nontemporal_store(s + 1, a.out_occ[1] + i);
+  __builtin_nontemporal_store((uint8_t)s, a.out_status + i);
 }
 
 struct Timer {
@@ -266,7 +248,6 @@ int hbt_measure_record_stream_gbps(int64_t n, int warmup, int launches, double* 
   using namespace hbt;
   if (n < 2 || n > ((int64_t)1 << 30) || warmup < 0 || launches <= 0 || out_gbps == nullptr)
     return HBT_EINVAL;
-  n &= ~(int64_t)1;
   // one allocation: 5 int32 + 4 fp64 input columns, fp64 + 2 int32 + 1 byte output columns
   const size_t col4 = ((size_t)n * 4 + 255) & ~(size_t)255, col8 = ((size_t)n * 8 + 255) & ~(size_t)255;
   const size_t total = 7 * col4 + 5 * col8 + (size_t)n;
@@ -284,17 +265,17 @@ int hbt_measure_record_stream_gbps(int64_t n, int warmup, int launches, double* 
   a.out_occ[1] = reinterpret_cast<int32_t*>(p); p += col4;
   a.out_status = reinterpret_cast<uint8_t*>(p);
   a.n = (uint32_t)n;
-  const unsigned blocks = (unsigned)((n / 2 + 63) / 64);
+  const unsigned blocks = (unsigned)((n + 127) / 128);
   Timer t;
   int rc = t.ok ? HBT_OK : HBT_EHIP;
   float ms = 0.f;
   if (rc == HBT_OK && hipMemsetAsync(base, 0, total, nullptr) != hipSuccess) rc = HBT_EHIP;
   if (rc == HBT_OK) {
     for (int i = 0; i < warmup; ++i)
-      hipLaunchKernelGGL(record_stream_kernel, dim3(blocks), dim3(64), 0, nullptr, a);
+      hipLaunchKernelGGL(record_stream_kernel, dim3(blocks), dim3(128), 0, nullptr, a);
     (void)hipEventRecord(t.e0, nullptr);
     for (int i = 0; i < launches; ++i)
-      hipLaunchKernelGGL(record_stream_kernel, dim3(blocks), dim3(64), 0, nullptr, a);
+      hipLaunchKernelGGL(record_stream_kernel, dim3(blocks), dim3(128), 0, nullptr, a);
     (void)hipEventRecord(t.e1, nullptr);
     if (hipEventSynchronize(t.e1) != hipSuccess ||
         hipEventElapsedTime(&ms, t.e0, t.e1) != hipSuccess || hipGetLastError() != hipSuccess)

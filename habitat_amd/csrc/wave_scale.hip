@@ -8,8 +8,9 @@
 // and the scaled time.
 //
 // Data layout: structure of arrays, one column per record field.  A thread owns
-// two consecutive records, so every int32 column is one 8-byte load per lane
-// and every fp64 column one 16-byte load; stores likewise.  All loads of a
+// kVectorRecords consecutive records (one, as measured best; the code is written
+// for any number), so a wavefront reads 256 contiguous bytes of every int32
+// column and 512 of every fp64 column; stores likewise.  All loads of a
 // thread are issued before any arithmetic and all stores after it, so that no
 // wait for a load also waits for a store.  Device constants travel in the
 // kernel-argument segment and live in SGPRs.  The algorithmic traffic is 52 B
@@ -35,11 +36,12 @@ namespace {
 using namespace dev;
 
 constexpr int kRecPerThread = kVectorRecords;
-// One wavefront per workgroup.  Measured at 1 M records under continuous
-// launches: 64 threads 11.7 us, 128 11.9, 256 12.5, 512 13.5 (and 512 was the
-// only size that ran faster, 12.3 us, for the first milliseconds after idle);
-// at 64 M records 64 threads are ahead as well (725 against 752-761 us).
-constexpr int kBlock = 64;
+// Two wavefronts per workgroup.  Measured under continuous launches with one
+// record per thread: 128 threads 11.7 us at 1 M records and 687 us at 64 M,
+// 64 threads 11.6 and 719, 256 threads 12.2 and 709.  (With two records per
+// thread: 64 threads 11.7 us, 128 11.9, 256 12.5, 512 13.5, and 512 was the only
+// size that ran faster, 12.3 us, for the first milliseconds after idle.)
+constexpr int kBlock = 128;
 
 // N consecutive elements as one register group (a scalar when N is 1).
 template <class T, int N>
