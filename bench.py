@@ -367,7 +367,7 @@ def main():
                      "traffic": TRAFFIC_BYTES_PER_RECORD * args.records,
                      "traffic_unit": "bytes/launch (FETCH_SIZE + WRITE_SIZE, rocprofv3, "
                                      "copy-calibrated; see profiles/)",
-                     "kernel": "wave_scale_kernel<1, true, true, unsigned int>", "launch_us": launch_ms * 1e3,
+                     "kernel": "wave_scale_kernel<1, 1, true, unsigned int>", "launch_us": launch_ms * 1e3,
                      "bytes_per_record": BYTES_PER_RECORD},
     }
 

@@ -80,6 +80,11 @@ struct OccDevice {
     return (flags & (kOk | kFastOk | kWarpPow2 | kCdna | kGp100 | kPoolSteps)) ==
            (kOk | kFastOk | kWarpPow2);
   }
+  // likewise for the compute-unit model: an accepted AMD description with
+  // small limits and a power-of-two wavefront size
+  HBT_HD bool cdna_lean_ok() const {
+    return (flags & (kOk | kFastOk | kWarpPow2 | kCdna)) == (kOk | kFastOk | kWarpPow2 | kCdna);
+  }
 };
 
 // Shared-memory pool a cc 7.x SM is configured to for an allocation of `size`
@@ -295,9 +300,12 @@ HBT_HD int32_t occupancy_fast(const OccDevice& d, int32_t block, const SmemAlloc
 // LDS per work-group beyond the limits, or a negative size).  There is no
 // counterpart in the reference.  `regs` is already narrowed to 16 bits.
 // EXACT_DIV: plain integer division (host; devices outside kFastOk).
-template <bool EXACT_DIV>
+// LEAN: the caller has checked cdna_lean_ok(), so the tests that are uniform
+// over a launch are not compiled in.
+template <bool EXACT_DIV, bool LEAN = false>
 HBT_HD int32_t occupancy_cdna(const OccDevice& d, int32_t block, int32_t smem_total, int32_t regs) {
-  if (!d.ok()) return 0;
+  static_assert(!(EXACT_DIV && LEAN), "the lean form is the 32-bit one");
+  if (!LEAN && !d.ok()) return 0;
   const bool in_range = block > 0 && block <= d.max_threads_per_block &&
                         regs <= d.vgprs_per_simd() && smem_total >= 0 &&
                         smem_total <= d.smem_per_block;
@@ -321,8 +329,8 @@ HBT_HD int32_t occupancy_cdna(const OccDevice& d, int32_t block, int32_t smem_to
     lim_lds = (int32_t)(d.smem_per_sm / (rounded > 0 ? rounded : 1));
   } else {
     const int32_t ws = d.warp_size;
-    const int32_t waves = (d.flags & kWarpPow2) ? ((block + ws - 1) >> d.warp_shift)
-                                                : fast_div(block + ws - 1, ws);
+    const int32_t waves = (LEAN || (d.flags & kWarpPow2)) ? ((block + ws - 1) >> d.warp_shift)
+                                                          : fast_div(block + ws - 1, ws);
     int32_t per_simd = fast_div(d.vgprs_per_simd(), alloc);
     per_simd = per_simd < slots_per_simd ? per_simd : slots_per_simd;
     lim = fast_div(per_simd << 2, waves);

@@ -36,7 +36,7 @@
 
 struct hbt_device_table {
   int32_t n_dest;
-  int32_t fast;            // every device (origin included) has lean_ok()
+  int32_t model;           // dev::kModel...: which occupancy models the kernel needs
   int device;
   hbt::OriginArgs origin;
   hbt::DestArgs* dests;    // device memory, [n_dest]
@@ -79,7 +79,7 @@ __global__ void fill_zero_kernel(double* sums, int64_t n_sums, int32_t* bad, int
 // One thread per (record, destination).  Within a wavefront, consecutive
 // records of the same segment are summed with a segmented scan and the last
 // lane of each run adds the run's total to the segment's sum.
-template <bool FAST>
+template <int MODEL>
 __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a) {
   const int d = blockIdx.y;
   const DestArgs& p = a.dests[d];
@@ -102,10 +102,10 @@ __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a)
   // lanes past the end form a run of their own so that they never swallow a tail
   const int32_t seg = in_range ? (a.segment != nullptr ? a.segment[j] : 0) : -1;
 
-  RecordMid m = origin_part<FAST>(a.origin, r);
+  RecordMid m = origin_part<MODEL != dev::kModelGeneral>(a.origin, r);
   if (__builtin_expect(m.redo_gflops, 0))
     m.num_gflops = origin_gflops_exact(a.origin.peak_gflops, r.eff, r.t);
-  const RecordOut o = dest_part<FAST, false>(p, r, m, 0.0);
+  const RecordOut o = dest_part<MODEL, false>(p, r, m, 0.0);
 
   const bool ok = in_range && o.status == HBT_ST_OK;
   double v = ok ? o.t : 0.0;
@@ -232,13 +232,14 @@ hbt_device_table* hbt_device_table_create(const hbt_device_spec* origin,
   t->n_dest = n_dest;
   t->device = device;
   t->origin = make_origin_args(*origin);
-  bool fast = t->origin.dev.lean_ok();
+  bool lean = t->origin.dev.lean_ok(), lean_cdna = lean;
   std::vector<DestArgs> host((size_t)n_dest);
   for (int32_t d = 0; d < n_dest; ++d) {
     host[d] = make_dest_args(*origin, dests[d]);
-    fast = fast && host[d].dev.lean_ok();
+    lean = lean && host[d].dev.lean_ok();
+    lean_cdna = lean_cdna && host[d].dev.cdna_lean_ok();
   }
-  t->fast = fast ? 1 : 0;
+  t->model = lean ? dev::kModelLean : lean_cdna ? dev::kModelLeanCdnaDest : dev::kModelGeneral;
   t->dests = nullptr;
   const size_t bytes = sizeof(DestArgs) * (size_t)n_dest;
   if (hipMalloc(reinterpret_cast<void**>(&t->dests), bytes) != hipSuccess) {
@@ -310,10 +311,14 @@ int hbt_wave_scale_sum(const hbt_device_table* table, int64_t n, const int32_t* 
   a.dests = table->dests;
   a.origin = table->origin;
   const dim3 grid((unsigned)blocks, (unsigned)table->n_dest);
-  if (table->fast)
-    hipLaunchKernelGGL(wave_scale_sum_kernel<true>, grid, dim3(kBlock), 0, stream, a);
+  if (table->model == dev::kModelLean)
+    hipLaunchKernelGGL(wave_scale_sum_kernel<dev::kModelLean>, grid, dim3(kBlock), 0, stream, a);
+  else if (table->model == dev::kModelLeanCdnaDest)
+    hipLaunchKernelGGL(wave_scale_sum_kernel<dev::kModelLeanCdnaDest>, grid, dim3(kBlock), 0,
+                       stream, a);
   else
-    hipLaunchKernelGGL(wave_scale_sum_kernel<false>, grid, dim3(kBlock), 0, stream, a);
+    hipLaunchKernelGGL(wave_scale_sum_kernel<dev::kModelGeneral>, grid, dim3(kBlock), 0, stream,
+                       a);
   return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
 }
 

@@ -94,7 +94,7 @@ __device__ __forceinline__ void store_r(T* __restrict__ p, Index i, const T (&in
 // SINGLE: the launch has one destination; its constants then sit at fixed
 // offsets of the argument segment and are fetched once, up front, instead of
 // inside a loop over destinations.
-template <int R, bool FAST, bool PERMUTE, bool SINGLE, class Index>
+template <int R, int MODEL, bool PERMUTE, bool SINGLE, class Index>
 __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
   const double log2_lane = PERMUTE ? kLog2Int[threadIdx.x & 63] : 0.0;
   int32_t nb[R], block[R], dyn[R], stat[R], regs[R], dregs[R];
@@ -132,7 +132,7 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
   for (int k = 0; k < R; ++k) {
     rin[k] = RecordIn{nb[k], block[k], smem_sum(stat[k], dyn[k]), regs[k], dregs[k],
                       true, t[k], eff[k], rd[k], wr[k]};
-    mid[k] = origin_part<FAST>(a.origin, rin[k]);
+    mid[k] = origin_part<MODEL != dev::kModelGeneral>(a.origin, rin[k]);
   }
   bool redo = false;
 #pragma unroll
@@ -157,7 +157,7 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
     uint8_t st[R];
 #pragma unroll
     for (int k = 0; k < R; ++k) {
-      const RecordOut o = dest_part<FAST, PERMUTE>(p, rin[k], mid[k], log2_lane);
+      const RecordOut o = dest_part<MODEL, PERMUTE>(p, rin[k], mid[k], log2_lane);
       ot[k] = o.t; occ_d[k] = o.occ_d; wave_d[k] = o.wave_d; st[k] = o.status;
     }
     const DestOut& w = a.out[d];
@@ -179,7 +179,7 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
   }
 }
 
-template <int R, bool FAST, bool SINGLE, class Index>
+template <int R, int MODEL, bool SINGLE, class Index>
 __global__ __launch_bounds__(kBlock) void wave_scale_kernel(const WaveScaleArgs a) {
   const Index thread = (Index)blockIdx.x * kBlock + threadIdx.x;
   const Index i = thread * R;
@@ -189,45 +189,52 @@ __global__ __launch_bounds__(kBlock) void wave_scale_kernel(const WaveScaleArgs 
   // record at a time.
   const Index wave_end = ((thread | 63) + 1) * R;
   if (wave_end <= n) {
-    process<R, FAST, true, SINGLE, Index>(a, i);
+    process<R, MODEL, true, SINGLE, Index>(a, i);
   } else {
     const Index end = (i + R < n) ? i + R : n;
-    for (Index j = i; j < end; ++j) process<1, FAST, false, SINGLE, Index>(a, j);
+    for (Index j = i; j < end; ++j) process<1, MODEL, false, SINGLE, Index>(a, j);
   }
 }
 
-template <int R, bool FAST, class Index>
+template <int R, int MODEL, class Index>
 void launch(const WaveScaleArgs& args, hipStream_t stream) {
   const int64_t threads = (args.n + R - 1) / R;
   const int64_t blocks = (threads + kBlock - 1) / kBlock;
   if (args.n_dest == 1)
-    hipLaunchKernelGGL((wave_scale_kernel<R, FAST, true, Index>), dim3((unsigned)blocks),
+    hipLaunchKernelGGL((wave_scale_kernel<R, MODEL, true, Index>), dim3((unsigned)blocks),
                        dim3(kBlock), 0, stream, args);
   else
-    hipLaunchKernelGGL((wave_scale_kernel<R, FAST, false, Index>), dim3((unsigned)blocks),
+    hipLaunchKernelGGL((wave_scale_kernel<R, MODEL, false, Index>), dim3((unsigned)blocks),
                        dim3(kBlock), 0, stream, args);
 }
 
-template <int R, bool FAST>
+template <int R, int MODEL>
 void launch(const WaveScaleArgs& args, hipStream_t stream) {
   // 32-bit byte offsets when the widest column (8 bytes per record) and the
   // thread numbering stay below 2^32 with room for the last wavefront.
-  if (args.n < ((int64_t)1 << 28)) launch<R, FAST, uint32_t>(args, stream);
-  else launch<R, FAST, uint64_t>(args, stream);
+  if (args.n < ((int64_t)1 << 28)) launch<R, MODEL, uint32_t>(args, stream);
+  else launch<R, MODEL, uint64_t>(args, stream);
 }
 
 }  // namespace
 
 hipError_t launch_wave_scale(const WaveScaleArgs& args, bool vectorised, hipStream_t stream) {
   if (args.n <= 0) return hipSuccess;
-  bool fast = args.origin.dev.lean_ok();
-  for (int d = 0; d < args.n_dest; ++d) fast = fast && args.dest[d].dev.lean_ok();
-  if (vectorised) {
-    if (fast) launch<kRecPerThread, true>(args, stream);
-    else launch<kRecPerThread, false>(args, stream);
-  } else {
-    if (fast) launch<1, true>(args, stream);
-    else launch<1, false>(args, stream);
+  bool lean = args.origin.dev.lean_ok(), lean_cdna = lean;
+  for (int d = 0; d < args.n_dest; ++d) {
+    lean = lean && args.dest[d].dev.lean_ok();
+    lean_cdna = lean_cdna && args.dest[d].dev.cdna_lean_ok();
+  }
+  const int model = lean ? dev::kModelLean
+                         : lean_cdna ? dev::kModelLeanCdnaDest : dev::kModelGeneral;
+  const bool vec = vectorised && kRecPerThread > 1;
+  switch (model * 2 + (vec ? 1 : 0)) {
+    case 0: launch<1, dev::kModelGeneral>(args, stream); break;
+    case 1: launch<kRecPerThread, dev::kModelGeneral>(args, stream); break;
+    case 2: launch<1, dev::kModelLean>(args, stream); break;
+    case 3: launch<kRecPerThread, dev::kModelLean>(args, stream); break;
+    case 4: launch<1, dev::kModelLeanCdnaDest>(args, stream); break;
+    default: launch<kRecPerThread, dev::kModelLeanCdnaDest>(args, stream); break;
   }
   return hipGetLastError();
 }

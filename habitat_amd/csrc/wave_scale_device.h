@@ -98,18 +98,29 @@ __device__ __forceinline__ bool div_const_safe(double x) {
 struct C100 { static constexpr double value = 100.0; };
 struct C1e9 { static constexpr double value = 1e9; };
 
-// FAST: the lean instantiation.  Every device of the launch has
-// OccDevice::lean_ok, so the 32-bit NVIDIA-rule model applies to every record
-// and nothing else is compiled in.  Otherwise each device picks its model by
-// wave-uniform branches: the compute-unit model for AMD descriptions, the
-// 64-bit model with real divisions for devices with limits of 2^20 and more
-// (not real hardware, but in the domain).
-template <bool FAST>
+// Which occupancy models a kernel instantiation contains.
+//   kModelLean: every device of the launch has OccDevice::lean_ok, so the
+//     32-bit NVIDIA-rule model applies to every record and nothing else is
+//     compiled in.
+//   kModelLeanCdnaDest: the origin has lean_ok and every destination
+//     cdna_lean_ok (a trace measured on an NVIDIA GPU, scaled to AMD
+//     descriptions): the same for the origin, the compute-unit model for the
+//     destinations, no uniform branches either.
+//   kModelGeneral: each device picks its model by wave-uniform branches: the
+//     compute-unit model for AMD descriptions, the 64-bit model with real
+//     divisions for devices with limits of 2^20 and more (not real hardware,
+//     but in the domain).
+// A bool converts: false is general, true is lean.
+enum : int { kModelGeneral = 0, kModelLean = 1, kModelLeanCdnaDest = 2 };
+
+template <int MODEL, bool DEST = false>
 __device__ __forceinline__ int32_t occupancy_dev(const OccDevice& d, int32_t block,
                                                  int32_t smem_total, const SmemAlloc& sm,
                                                  int32_t regs) {
   regs &= 0xFFFF;  // uint16_t narrowing, cpp/src/cuda/kernel.h:108
-  if (FAST) return occupancy_fast<true>(d, block, sm, regs);
+  if (MODEL == kModelLeanCdnaDest && DEST)
+    return occupancy_cdna<false, true>(d, block, smem_total, regs);
+  if (MODEL != kModelGeneral) return occupancy_fast<true>(d, block, sm, regs);
   if (d.flags & kCdna)
     return d.fast_ok() ? occupancy_cdna<false>(d, block, smem_total, regs)
                        : occupancy_cdna<true>(d, block, smem_total, regs);
@@ -204,12 +215,12 @@ __device__ __forceinline__ double roofline_gamma(const DestArgs& p, double num_g
   return (num_gflops < 1e-9 || !metrics) ? 1. : gamma;
 }
 
-template <bool FAST, bool PERMUTE>
+template <int MODEL, bool PERMUTE>
 __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn& r,
                                                const RecordMid& m, double log2_lane) {
   RecordOut o;
   const int32_t regs_d = r.dest_regs >= 0 ? r.dest_regs : r.regs;
-  o.occ_d = occupancy_dev<FAST>(p.dev, r.block, r.smem_total, m.smem, regs_d);
+  o.occ_d = occupancy_dev<MODEL, true>(p.dev, r.block, r.smem_total, m.smem, regs_d);
   o.wave_d = mul_small(p.dev.num_sms, o.occ_d);
 
   const double gamma = roofline_gamma(p, m.num_gflops, m.total_gb, r.metrics);
@@ -218,7 +229,8 @@ __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn
   // `a // wave_o == 0 and a // wave_d == 0`: the second test, and its division
   // by zero, happen only when the first holds (roofline.py:29-30).
   const bool small = m.small_o && r.nb < o.wave_d;
-  const int32_t dest_max_occ = ceil_div_small<FAST>(small ? r.nb : 0, p.dev.num_sms, p.inv_sms);
+  const int32_t dest_max_occ =
+      ceil_div_small<MODEL != kModelGeneral>(small ? r.nb : 0, p.dev.num_sms, p.inv_sms);
 
   int32_t status = HBT_ST_OK;
   status = (r.metrics && small && m.origin_max_occ == 0) ? HBT_ST_ZERO_BLOCKS : status;
