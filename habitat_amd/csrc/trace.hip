@@ -102,7 +102,7 @@ __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a)
   // lanes past the end form a run of their own so that they never swallow a tail
   const int32_t seg = in_range ? (a.segment != nullptr ? a.segment[j] : 0) : -1;
 
-  RecordMid m = origin_part<MODEL != dev::kModelGeneral>(a.origin, r);
+  RecordMid m = origin_part<MODEL>(a.origin, r);
   if (__builtin_expect(m.redo_gflops, 0))
     m.num_gflops = origin_gflops_exact(a.origin.peak_gflops, r.eff, r.t);
   const RecordOut o = dest_part<MODEL, false>(p, r, m, 0.0);
@@ -232,14 +232,14 @@ hbt_device_table* hbt_device_table_create(const hbt_device_spec* origin,
   t->n_dest = n_dest;
   t->device = device;
   t->origin = make_origin_args(*origin);
-  bool lean = t->origin.dev.lean_ok(), lean_cdna = lean;
+  bool lean = true, cdna = true;
   std::vector<DestArgs> host((size_t)n_dest);
   for (int32_t d = 0; d < n_dest; ++d) {
     host[d] = make_dest_args(*origin, dests[d]);
     lean = lean && host[d].dev.lean_ok();
-    lean_cdna = lean_cdna && host[d].dev.cdna_lean_ok();
+    cdna = cdna && host[d].dev.cdna_lean_ok();
   }
-  t->model = lean ? dev::kModelLean : lean_cdna ? dev::kModelLeanCdnaDest : dev::kModelGeneral;
+  t->model = dev::model_for(t->origin.dev.lean_ok(), t->origin.dev.cdna_lean_ok(), lean, cdna);
   t->dests = nullptr;
   const size_t bytes = sizeof(DestArgs) * (size_t)n_dest;
   if (hipMalloc(reinterpret_cast<void**>(&t->dests), bytes) != hipSuccess) {
@@ -311,14 +311,9 @@ int hbt_wave_scale_sum(const hbt_device_table* table, int64_t n, const int32_t* 
   a.dests = table->dests;
   a.origin = table->origin;
   const dim3 grid((unsigned)blocks, (unsigned)table->n_dest);
-  if (table->model == dev::kModelLean)
-    hipLaunchKernelGGL(wave_scale_sum_kernel<dev::kModelLean>, grid, dim3(kBlock), 0, stream, a);
-  else if (table->model == dev::kModelLeanCdnaDest)
-    hipLaunchKernelGGL(wave_scale_sum_kernel<dev::kModelLeanCdnaDest>, grid, dim3(kBlock), 0,
-                       stream, a);
-  else
-    hipLaunchKernelGGL(wave_scale_sum_kernel<dev::kModelGeneral>, grid, dim3(kBlock), 0, stream,
-                       a);
+  dev::with_model(table->model, [&](auto m) {
+    hipLaunchKernelGGL(wave_scale_sum_kernel<decltype(m)::value>, grid, dim3(kBlock), 0, stream, a);
+  });
   return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
 }
 

@@ -132,7 +132,7 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
   for (int k = 0; k < R; ++k) {
     rin[k] = RecordIn{nb[k], block[k], smem_sum(stat[k], dyn[k]), regs[k], dregs[k],
                       true, t[k], eff[k], rd[k], wr[k]};
-    mid[k] = origin_part<MODEL != dev::kModelGeneral>(a.origin, rin[k]);
+    mid[k] = origin_part<MODEL>(a.origin, rin[k]);
   }
   bool redo = false;
 #pragma unroll
@@ -220,22 +220,18 @@ void launch(const WaveScaleArgs& args, hipStream_t stream) {
 
 hipError_t launch_wave_scale(const WaveScaleArgs& args, bool vectorised, hipStream_t stream) {
   if (args.n <= 0) return hipSuccess;
-  bool lean = args.origin.dev.lean_ok(), lean_cdna = lean;
+  bool lean = true, cdna = true;
   for (int d = 0; d < args.n_dest; ++d) {
     lean = lean && args.dest[d].dev.lean_ok();
-    lean_cdna = lean_cdna && args.dest[d].dev.cdna_lean_ok();
+    cdna = cdna && args.dest[d].dev.cdna_lean_ok();
   }
-  const int model = lean ? dev::kModelLean
-                         : lean_cdna ? dev::kModelLeanCdnaDest : dev::kModelGeneral;
+  const int model =
+      model_for(args.origin.dev.lean_ok(), args.origin.dev.cdna_lean_ok(), lean, cdna);
   const bool vec = vectorised && kRecPerThread > 1;
-  switch (model * 2 + (vec ? 1 : 0)) {
-    case 0: launch<1, dev::kModelGeneral>(args, stream); break;
-    case 1: launch<kRecPerThread, dev::kModelGeneral>(args, stream); break;
-    case 2: launch<1, dev::kModelLean>(args, stream); break;
-    case 3: launch<kRecPerThread, dev::kModelLean>(args, stream); break;
-    case 4: launch<1, dev::kModelLeanCdnaDest>(args, stream); break;
-    default: launch<kRecPerThread, dev::kModelLeanCdnaDest>(args, stream); break;
-  }
+  with_model(model, [&](auto m) {
+    if (vec) launch<kRecPerThread, decltype(m)::value>(args, stream);
+    else launch<1, decltype(m)::value>(args, stream);
+  });
   return hipGetLastError();
 }
 

@@ -13,6 +13,7 @@
 
 #include <cmath>
 #include <cstdint>
+#include <type_traits>
 
 #include "occupancy.h"
 #include "wave_scale.h"
@@ -99,27 +100,54 @@ struct C100 { static constexpr double value = 100.0; };
 struct C1e9 { static constexpr double value = 1e9; };
 
 // Which occupancy models a kernel instantiation contains.
-//   kModelLean: every device of the launch has OccDevice::lean_ok, so the
-//     32-bit NVIDIA-rule model applies to every record and nothing else is
-//     compiled in.
-//   kModelLeanCdnaDest: the origin has lean_ok and every destination
-//     cdna_lean_ok (a trace measured on an NVIDIA GPU, scaled to AMD
-//     descriptions): the same for the origin, the compute-unit model for the
-//     destinations, no uniform branches either.
+//   The four lean ones: the origin and every destination of the launch have
+//     OccDevice::lean_ok (the 32-bit NVIDIA-rule model, straight-line) or
+//     cdna_lean_ok (the compute-unit model, straight-line), the origin one kind
+//     and the destinations all one kind; nothing else is compiled in and no
+//     branch is uniform over the launch.
 //   kModelGeneral: each device picks its model by wave-uniform branches: the
 //     compute-unit model for AMD descriptions, the 64-bit model with real
 //     divisions for devices with limits of 2^20 and more (not real hardware,
 //     but in the domain).
-// A bool converts: false is general, true is lean.
-enum : int { kModelGeneral = 0, kModelLean = 1, kModelLeanCdnaDest = 2 };
+enum : int {
+  kModelGeneral = 0,
+  kModelLean = 1,            // NVIDIA-rule origin and destinations
+  kModelLeanCdnaDest = 2,    // NVIDIA-rule origin, AMD destinations
+  kModelLeanCdnaOrigin = 3,  // AMD origin, NVIDIA-rule destinations
+  kModelLeanCdna = 4,        // AMD origin and destinations
+};
 
-template <int MODEL, bool DEST = false>
+// The instantiation for a launch whose origin and destinations are of these
+// kinds (each: lean_ok, cdna_lean_ok, or neither).
+inline int model_for(bool origin_lean, bool origin_cdna_lean, bool dests_lean,
+                     bool dests_cdna_lean) {
+  if (origin_lean && dests_lean) return kModelLean;
+  if (origin_lean && dests_cdna_lean) return kModelLeanCdnaDest;
+  if (origin_cdna_lean && dests_lean) return kModelLeanCdnaOrigin;
+  if (origin_cdna_lean && dests_cdna_lean) return kModelLeanCdna;
+  return kModelGeneral;
+}
+
+// Calls f with the model as a compile-time constant.
+template <class F>
+inline void with_model(int model, F&& f) {
+  switch (model) {
+    case kModelLean: f(std::integral_constant<int, kModelLean>()); break;
+    case kModelLeanCdnaDest: f(std::integral_constant<int, kModelLeanCdnaDest>()); break;
+    case kModelLeanCdnaOrigin: f(std::integral_constant<int, kModelLeanCdnaOrigin>()); break;
+    case kModelLeanCdna: f(std::integral_constant<int, kModelLeanCdna>()); break;
+    default: f(std::integral_constant<int, kModelGeneral>()); break;
+  }
+}
+
+template <int MODEL, bool DEST>
 __device__ __forceinline__ int32_t occupancy_dev(const OccDevice& d, int32_t block,
                                                  int32_t smem_total, const SmemAlloc& sm,
                                                  int32_t regs) {
   regs &= 0xFFFF;  // uint16_t narrowing, cpp/src/cuda/kernel.h:108
-  if (MODEL == kModelLeanCdnaDest && DEST)
-    return occupancy_cdna<false, true>(d, block, smem_total, regs);
+  constexpr bool cdna = DEST ? (MODEL == kModelLeanCdnaDest || MODEL == kModelLeanCdna)
+                             : (MODEL == kModelLeanCdnaOrigin || MODEL == kModelLeanCdna);
+  if (cdna) return occupancy_cdna<false, true>(d, block, smem_total, regs);
   if (MODEL != kModelGeneral) return occupancy_fast<true>(d, block, sm, regs);
   if (d.flags & kCdna)
     return d.fast_ok() ? occupancy_cdna<false>(d, block, smem_total, regs)
@@ -141,15 +169,15 @@ __device__ __forceinline__ int32_t ceil_div_small(int32_t nb, int32_t sms, float
   return (int32_t)(((int64_t)nb + sms - 1) / sms);
 }
 
-template <bool FAST>
+template <int MODEL>
 __device__ __forceinline__ RecordMid origin_part(const OriginArgs& o, const RecordIn& r) {
   RecordMid m;
   m.smem = smem_alloc(r.smem_total);
-  m.occ_o = occupancy_dev<FAST>(o.dev, r.block, r.smem_total, m.smem, r.regs);
+  m.occ_o = occupancy_dev<MODEL, false>(o.dev, r.block, r.smem_total, m.smem, r.regs);
   m.wave_o = mul_small(o.dev.num_sms, m.occ_o);
   m.small_o = r.nb >= 0 && r.nb < m.wave_o;
   m.origin_max_occ =
-      ceil_div_small<FAST>(m.small_o ? r.nb : 0, o.dev.num_sms, o.inv_sms);
+      ceil_div_small<MODEL != kModelGeneral>(m.small_o ? r.nb : 0, o.dev.num_sms, o.inv_sms);
   // roofline.py:72-76, same operation order.  The three divisions by 1024 are
   // exact scalings, done here as one by 2^-30.  (Below 2^-992 bytes, where a
   // quotient is subnormal and one rounding is not three, the last bits of

@@ -184,46 +184,52 @@ def test_strategy_and_sweep_use_the_compute_unit_model():
 
 
 @pytest.mark.gpu
-def test_lean_and_general_instantiations_agree_bit_for_bit_for_amd_destinations():
-    """An NVIDIA origin with AMD destinations only runs a kernel instantiation
-    without the model's uniform branches; a P100 among the destinations forces
-    the general one.  Same records, same AMD destination: every output of that
-    destination must be identical, on ordinary records and on field values at
-    and beyond the limits, and the occupancies must be the host routine's."""
+@pytest.mark.parametrize("case", ["nvidia_to_amd", "amd_to_nvidia", "amd_to_amd"])
+def test_lean_and_general_instantiations_agree_bit_for_bit(case):
+    """A launch whose origin and destinations are each of one kind (NVIDIA-rule
+    or AMD description) runs a kernel instantiation without the model's uniform
+    branches; a P100 among the destinations forces the general one.  Same
+    records, same first destination: every output of that destination must be
+    identical, on ordinary records and on field values at and beyond the limits,
+    and the occupancies must be the host routine's."""
+    import torch
     from test_wave_scale_gpu import adversarial_records
-    from habitat_amd.analysis.wave_scaling.batch import KernelRecords, wave_scale
     from habitat_amd import DeviceProperties
+    from habitat_amd.analysis.wave_scaling.batch import (DeviceTable, KernelRecords, wave_scale,
+                                                         wave_scale_sum)
     amd = Device.MI355X_cdna
     # a second AMD description: gfx942-like (64 KiB LDS, 512-byte granules, 304 CUs)
-    other = DeviceProperties(name="other", **dict(
+    amd2 = DeviceProperties(name="other", **dict(
         amd.as_dict(), compute_minor=2, shared_mem_per_block=65536,
         shared_mem_per_multiprocessor=65536, num_sms=304, mem_bandwidth_gb=5300,
         base_clock_mhz=2100, peak_gflops_per_second=163400))
+    origin, first, other = {"nvidia_to_amd": (Device.V100, amd, amd2),
+                            "amd_to_nvidia": (amd, Device.V100, Device.T4),
+                            "amd_to_amd": (amd2, amd, amd2)}[case]
     ordinary, _ = synthetic.kernel_records(50_001, Device.V100, seed=5, metrics_fraction=0.8)
     for rec in (ordinary, adversarial_records(40_003, 17)):
         kr = KernelRecords.from_numpy(rec)
-        lean = wave_scale(kr, Device.V100, [amd, other], waves=True)
-        general = wave_scale(kr, Device.V100, [amd, Device.P100], waves=True)
-        single = wave_scale(kr, Device.V100, [amd], waves=True)
+        lean = wave_scale(kr, origin, [first, other], waves=True)
+        general = wave_scale(kr, origin, [first, Device.P100], waves=True)
+        single = wave_scale(kr, origin, [first], waves=True)
         for out in (lean, single):
             for name in ("time_ns", "occ_dest", "wave_dest", "status"):
                 a = getattr(out, name)[0].cpu().numpy()
                 b = getattr(general, name)[0].cpu().numpy()
                 assert np.array_equal(a, b, equal_nan=True), name
             assert np.array_equal(out.occ_origin.cpu().numpy(), general.occ_origin.cpu().numpy())
-        for d, dev in enumerate((amd, other)):
+        assert np.array_equal(lean.occ_origin.cpu().numpy(), host_batch(origin, rec))
+        for d, dev in enumerate((first, other)):
             asked = dict(rec)
             if "dest_regs" in rec:
                 asked["regs_per_thread"] = np.where(rec["dest_regs"] >= 0, rec["dest_regs"],
                                                     rec["regs_per_thread"])
             assert np.array_equal(lean.occ_dest[d].cpu().numpy(), host_batch(dev, asked))
-        # the per-segment sums take the same three instantiations
-        from habitat_amd.analysis.wave_scaling.batch import DeviceTable, wave_scale_sum
-        import torch
+        # the per-segment sums take the same instantiations
         seg = torch.arange(kr.n, dtype=torch.int32, device=kr.device) // 1000
         n_seg = (kr.n + 999) // 1000
-        sums_lean, bad_lean = wave_scale_sum(kr, DeviceTable(Device.V100, [amd, other]), seg, n_seg)
-        sums_gen, bad_gen = wave_scale_sum(kr, DeviceTable(Device.V100, [amd, Device.P100]), seg,
+        sums_lean, bad_lean = wave_scale_sum(kr, DeviceTable(origin, [first, other]), seg, n_seg)
+        sums_gen, bad_gen = wave_scale_sum(kr, DeviceTable(origin, [first, Device.P100]), seg,
                                            n_seg)
         assert torch.equal(bad_lean[0], bad_gen[0])
         a, b = sums_lean[0].cpu().numpy(), sums_gen[0].cpu().numpy()
