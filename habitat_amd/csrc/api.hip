@@ -117,12 +117,19 @@ int hbt_occupancy_host_model32_batch(const hbt_device_spec* spec, int64_t n,
   if (!hbt::occupancy_spec_in_domain(*spec)) return HBT_ESPEC;
   const hbt::OccDevice d = hbt::make_occ_device(*spec);
   if (!d.fast_ok()) return HBT_ESPEC;
+  // the form the kernels run for this device: the straight-line one where the
+  // device allows it
+  const bool lean = d.lean_ok(), cdna_lean = d.cdna_lean_ok();
   for (int64_t i = 0; i < n; ++i) {
     const int32_t smem_total = hbt::smem_sum(static_smem[i], dynamic_smem[i]);
-    out[i] = (d.flags & hbt::kCdna)
-                 ? hbt::occupancy_cdna<false>(d, block_size[i], smem_total, regs[i] & 0xFFFF)
-                 : hbt::occupancy_fast<false>(d, block_size[i], hbt::smem_alloc(smem_total),
-                                       regs[i] & 0xFFFF);
+    const int32_t r = regs[i] & 0xFFFF;
+    const int32_t b = block_size[i];
+    if (d.flags & hbt::kCdna)
+      out[i] = cdna_lean ? hbt::occupancy_cdna<false, true>(d, b, smem_total, r)
+                         : hbt::occupancy_cdna<false>(d, b, smem_total, r);
+    else
+      out[i] = lean ? hbt::occupancy_fast<true>(d, b, hbt::smem_alloc(smem_total), r)
+                    : hbt::occupancy_fast<false>(d, b, hbt::smem_alloc(smem_total), r);
   }
   return HBT_OK;
 }

@@ -115,7 +115,8 @@ int hbt_occupancy_host_batch(const hbt_device_spec *spec, int64_t n, const int32
  * Diagnostic: the 32-bit formulation of the same model that the wave-scaling
  * kernel uses for devices whose limits are all below 2^20, evaluated on the
  * HOST over host arrays (its float-reciprocal divisions replaced by exact
- * ones).  Lets the kernel's integer logic be checked against
+ * ones), in the straight-line form the kernels run where the device allows
+ * it.  Lets the kernel's integer logic be checked against
  * hbt_occupancy_host_batch without a GPU.  Returns HBT_ESPEC for a device
  * outside that formulation's domain.  No counterpart in the reference.
  */
