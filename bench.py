@@ -166,7 +166,7 @@ def mlp_bench(args):
                       "the first %d rows, %d torch threads" % (m, threads)}
     # few rows: the reference's own call pattern is one row per call (mlp.py:252-267)
     few = {}
-    for rows in (1, 108, 512):
+    for rows in (1, 108, 512, 4096):
         xs = xg[:rows].contiguous()
         ys = torch.empty(rows, dtype=torch.float32, device="cuda")
         _, f_launch = time_steps(lambda: rp.predict_batch(xs, out=ys), 50, 5)
@@ -179,7 +179,7 @@ def mlp_bench(args):
         for i in range(20):
             omlp.forward_fp32(sd, x[i:i + 1], mu, sigma)
         few["cpu_rows_1_us"] = (time.perf_counter() - t0) / 20 * 1e6
-    few["note"] = ("up to 512 rows: one launch per layer over the whole GPU (mlp_layer_kernel); "
+    few["note"] = ("up to 4096 rows: one launch per layer over the whole GPU (mlp_layer_kernel); "
                    "cpu_rows_1_us: torch CPU fp32, batch 1, as the reference predicts")
     mlp["few_rows"] = few
     others = {}

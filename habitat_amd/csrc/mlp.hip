@@ -41,6 +41,7 @@ namespace hbt {
 
 namespace {
 
+using f32x2 = float __attribute__((ext_vector_type(2)));
 using f32x4 = float __attribute__((ext_vector_type(4)));
 using f32x16 = float __attribute__((ext_vector_type(16)));
 
@@ -239,22 +240,31 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
 }
 
 // ---------------------------------------------------------------------------
-// Few rows (one prediction, the operations of one trace): one launch per layer.
+// Up to a few thousand rows (one prediction, the operations of one trace, a
+// trace for a handful of devices): one launch per layer.
 //
 // The fused kernel gives each workgroup 32 rows and the whole network, so a
 // batch of up to 32 rows runs on ONE compute unit, which has to pull all
-// 33.6 MB of weights through by itself (about 1 ms).  Here a layer is spread
-// over the chip instead: a workgroup takes NT n-tiles x one eighth of K x one
-// m-tile, its four waves split that K range again and add their 32 x 32
-// accumulators through LDS, and the eight K-partials of a layer are written to
-// a scratch buffer, [split][row][n].  They are summed, biased and rectified by
-// whoever reads them: the next layer's activation load, or the final dot
-// product.  The order of every sum is fixed, so results are reproducible.
-// Same packed weights, same MFMA instruction, same fragment layout as above.
-constexpr int kSplit = 8;            // K-partials per hidden layer
-constexpr int kSmallMaxRows = 512;   // largest batch that takes this path
-constexpr int kGroupsPerWave = (kWidth / 8) / kSplit / 4;  // 4 k-groups of a hidden layer
-static_assert(kGroupsPerWave == 4, "a wave of a hidden layer's workgroup owns four k-groups");
+// 33.6 MB of weights through by itself (about 1 ms), and any batch below 8192
+// rows leaves compute units idle for that long.  Here a layer is spread over
+// the chip instead: a workgroup takes one n-tile x one m-tile, its waves split
+// K, each issues the loads of all its k-groups at once, multiplies them as
+// they arrive and the waves add their 32 x 32 accumulators through LDS.
+//
+//   33 rows and more: eight waves cover all of K (16 k-groups each), the
+//   workgroup applies bias and ReLU and writes activations, [row][n].
+//   Up to 32 rows that would be 32 workgroups per layer, so K is split kSplit
+//   ways over workgroups as well (four waves, 4 k-groups each) and the
+//   K-partials are written as they are, [split][row][n]; they are summed,
+//   biased and rectified by whoever reads them: the next layer's activation
+//   load, or the final dot product.
+//
+// The order of every sum is fixed, so results are reproducible.  Same packed
+// weights, same MFMA instruction, same fragment layout as above.
+constexpr int kSplit = 8;            // K-partials per hidden layer, up to kRows rows
+constexpr int kLayerMaxRows = 4096;  // largest batch that takes this path
+constexpr size_t kScratchFloats = (size_t)kLayerMaxRows * kWidth;  // each of two buffers
+static_assert((size_t)kSplit * kRows * kWidth <= kScratchFloats, "the K-partials fit the scratch");
 
 struct LayerArgs {
   const float* w_stream;   // packed weights, see above
@@ -262,111 +272,154 @@ struct LayerArgs {
   int32_t g0;              // first stream group of this layer
   int32_t kg;              // k-groups of this layer (K / 8)
   int32_t splits;          // K-partials this launch writes (gridDim.y)
-  const float* p_in;       // [s_in][m_pad][kWidth], partials of the previous layer
-  int32_t s_in;
-  const float* bias_in;    // [kWidth], bias of the previous layer
+  const float* p_in;       // [m_pad][kWidth] activations, or [kSplit][m_pad][kWidth] partials
+  const float* bias_in;    // [kWidth], bias of the previous layer (with partials)
+  const float* bias_out;   // [kWidth], bias of this layer (FINAL)
   const double* raw;       // FIRST: [n][in_features], with mu and sigma
   const double* mu;
   const double* sigma;
   int32_t in_features;
   int64_t n;
   int32_t m_pad;           // rows rounded up to 32
-  float* p_out;            // [splits][m_pad][kWidth]
+  float* p_out;            // [m_pad][kWidth] activations (FINAL), else [splits][m_pad][kWidth]
 };
 
-// S_IN: K-partials of the input (1 after fc1, kSplit after a hidden layer); a
-// compile-time count so that all of a lane's partial loads are in flight at once.
-template <int NT, bool FIRST, int S_IN>
-__global__ __launch_bounds__(256) void mlp_layer_kernel(const LayerArgs a) {
-  __shared__ float red[4][NT][16][64];
+// G k-groups of a wave: the weight fragments of the n-tile and what the
+// matching activation fragments are made from (the activations themselves, or
+// S_IN K-partials and the bias that goes with them).
+template <int G, int S_IN>
+struct LayerFrag {
+  f32x4 w[G];
+  f32x4 x[G][S_IN > 0 ? S_IN : 1];
+  f32x4 bias[S_IN > 0 ? G : 1];
+};
+
+// One layer for one m-tile (blockIdx.z), one n-tile (blockIdx.x) and one
+// K-partial (blockIdx.y of a.splits).  The WAVES waves split the partial's
+// k-groups (at most G each); fc1 has fewer, so there each group is checked
+// against the wave's count (wave-uniform).
+//   FIRST: fc1, from the raw fp64 rows, standardised on the spot.
+//   S_IN: 0 = the input holds activations; kSplit = it holds that many
+//     K-partials, to be summed, biased and rectified on the way in.
+//   FINAL: the launch covers all of K (a.splits == 1), so the output is
+//     biased and rectified here and the next layer reads activations.
+//   PADDED_ROWS: rows past the end of the batch are read like the others (the
+//     padded m-tile holds them) instead of being masked; masking saves most of
+//     the traffic of a handful of rows, not masking keeps the loads of a full
+//     tile free of branches.
+template <bool FIRST, int S_IN, bool FINAL, int WAVES, bool PADDED_ROWS>
+__global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a) {
+  static_assert(S_IN == 0 || !FINAL, "K-partials go in and come out together");
+  static_assert(WAVES == 4 || WAVES == 8, "the reduction below is written for these");
+  constexpr int G = FIRST ? kMaxInPadded / 8 / WAVES : kWidth / 8 / WAVES / (FINAL ? 1 : kSplit);
+  __shared__ float red[WAVES][16][64];
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int m = lane & 31, h = lane >> 5;
   const int split = blockIdx.y;
+  // rows past the end of the batch: computed (from zeros, or from what the
+  // padded m-tile holds) and stored within the padded m-tile, never read out
   const int64_t row = (int64_t)blockIdx.z * kRows + m;
-  const bool row_ok = row < a.n;
+  const bool row_ok = PADDED_ROWS || row < a.n;
 
   // this wave's k-groups: [first, first + count) of the layer's kg
   const int per_split = a.kg / a.splits;
-  const int per_wave = (per_split + 3) / 4;
+  const int per_wave = (per_split + WAVES - 1) / WAVES;
   const int first = split * per_split + wave * per_wave;
   int count = per_split - wave * per_wave;
   count = count < 0 ? 0 : (count > per_wave ? per_wave : count);
 
-  f32x4 w[kGroupsPerWave][NT], x[kGroupsPerWave];
+  // n-tile of the layer -> (stream of the fused kernel's wave, slot in its group)
+  const int tile = blockIdx.x;
+  const f32x4* w_lane = reinterpret_cast<const f32x4*>(a.w_stream) +
+                        ((size_t)(tile >> 3) * a.groups_total + a.g0) * (8 * 64) +
+                        (tile & 7) * 64 + lane;
+
+  // every load of the wave, then the arithmetic in the order of arrival
+  const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+  LayerFrag<G, S_IN> f;
 #pragma unroll
-  for (int j = 0; j < kGroupsPerWave; ++j) {
-    const bool on = j < count;
-    const int gl = first + (on ? j : 0);  // layer-local group
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const int tile = blockIdx.x * NT + t;               // n-tile of the layer, 0..31
-      const int owner = tile >> 3, slot = tile & 7;       // stream of the fused kernel's wave
-      const f32x4* p = reinterpret_cast<const f32x4*>(a.w_stream) +
-                       ((size_t)owner * a.groups_total + a.g0 + gl) * (8 * 64) + slot * 64 + lane;
-      w[j][t] = on ? *p : f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-    const int k = 8 * gl + 4 * h;
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    if (on && row_ok) {
+  for (int j = 0; j < G; ++j) {
+    if (!FIRST || j < count) {
+      const int gl = first + j;  // layer-local group
+      f.w[j] = w_lane[(size_t)gl * (8 * 64)];
+      const int k = 8 * gl + 4 * h;
       if (FIRST) {
+        f32x4 v = zero;
+        if (row_ok) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (k + e < a.in_features)
-            v[e] = (float)((a.raw[row * a.in_features + k + e] - a.mu[k + e]) / a.sigma[k + e]);
+          for (int e = 0; e < 4; ++e)
+            if (k + e < a.in_features)
+              v[e] = (float)((a.raw[row * a.in_features + k + e] - a.mu[k + e]) / a.sigma[k + e]);
+        }
+        f.x[j][0] = v;
+      } else if (S_IN == 0) {
+        f.x[j][0] = zero;
+        if (row_ok) f.x[j][0] = *reinterpret_cast<const f32x4*>(a.p_in + (size_t)row * kWidth + k);
       } else {
-        f32x4 part[S_IN];
 #pragma unroll
-        for (int s = 0; s < S_IN; ++s)
-          part[s] = *reinterpret_cast<const f32x4*>(a.p_in + ((size_t)s * a.m_pad + row) * kWidth + k);
-        v = *reinterpret_cast<const f32x4*>(a.bias_in + k);
+        for (int s = 0; s < S_IN; ++s) f.x[j][s] = zero;
+        if (row_ok) {
 #pragma unroll
-        for (int s = 0; s < S_IN; ++s) v += part[s];
+          for (int s = 0; s < S_IN; ++s)
+            f.x[j][s] = *reinterpret_cast<const f32x4*>(a.p_in + ((size_t)s * a.m_pad + row) * kWidth + k);
+        }
+        f.bias[j] = *reinterpret_cast<const f32x4*>(a.bias_in + k);
+      }
+    }
+  }
+
+  f32x16 acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+  for (int j = 0; j < G; ++j) {
+    if (!FIRST || j < count) {
+      f32x4 v = f.x[j][0];
+      if (S_IN > 0) {
+        // the previous layer's K-partials, in their fixed order, then bias and ReLU
+        v = f.bias[j];
+#pragma unroll
+        for (int s = 0; s < S_IN; ++s) v += f.x[j][s];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = fmaxf(v[e], 0.f);
       }
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(f.w[j][e], v[e], acc, 0, 0, 0);
     }
-    x[j] = v;
   }
 
-  f32x16 acc[NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
-#pragma unroll
-  for (int j = 0; j < kGroupsPerWave; ++j)
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(w[j][t][e], x[j][e], acc[t], 0, 0, 0);
-
-#pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) red[wave][t][r][lane] = acc[t][r];
+  for (int r = 0; r < 16; ++r) red[wave][r][lane] = acc[r];
   __syncthreads();
-  // thread (q = wave, lane) adds the four waves' registers 4q..4q+3: accumulator
-  // register 4g + e of lane (m, h) is output n = 8g + 4h + e of row m
-  const int q = wave;
+  // thread (wave, lane) adds the waves' registers R*wave .. R*wave+R-1, in wave
+  // order: accumulator register 4g + e of lane (m, h) is output n = 8g + 4h + e
+  // of row m
+  constexpr int R = 16 / WAVES;
+  const int r0 = R * wave;
+  const int n0 = tile * 32 + 8 * (r0 >> 2) + 4 * h + (r0 & 3);
+  float o[R];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    f32x4 o;
+  for (int e = 0; e < R; ++e) {
+    float sum = red[0][r0 + e][lane];
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-      o[e] = ((red[0][t][4 * q + e][lane] + red[1][t][4 * q + e][lane]) +
-              red[2][t][4 * q + e][lane]) + red[3][t][4 * q + e][lane];
-    const int n0 = (blockIdx.x * NT + t) * 32 + 8 * q + 4 * h;
-    float* dst = a.p_out + ((size_t)split * a.m_pad + (size_t)blockIdx.z * kRows + m) * kWidth + n0;
-    *reinterpret_cast<f32x4*>(dst) = o;
+    for (int w = 1; w < WAVES; ++w) sum += red[w][r0 + e][lane];
+    if (FINAL) sum = fmaxf(sum + a.bias_out[n0 + e], 0.f);
+    o[e] = sum;
+  }
+  float* dst = a.p_out + ((size_t)split * a.m_pad + (size_t)blockIdx.z * kRows + m) * kWidth + n0;
+  if constexpr (R == 4) {
+    *reinterpret_cast<f32x4*>(dst) = f32x4{o[0], o[1], o[2], o[3]};
+  } else {
+    *reinterpret_cast<f32x2*>(dst) = f32x2{o[0], o[1]};
   }
 }
 
 struct LastArgs {
-  const float* p_in;     // [s_in][m_pad][kWidth]
-  int32_t s_in;
-  const float* bias_in;  // [kWidth]
+  const float* p_in;     // [m_pad][kWidth] activations, or [kSplit][m_pad][kWidth] partials
+  const float* bias_in;  // [kWidth], bias of the last hidden layer (with partials)
   const float* w_last;   // [kWidth]
   float b_last;
   int64_t n;
@@ -374,29 +427,35 @@ struct LastArgs {
   float* out;            // [n]
 };
 
-// fc2 for few rows: one wavefront per row.
+// fc2 for few rows: one wavefront per row.  S_IN as in mlp_layer_kernel.
 template <int S_IN>
 __global__ __launch_bounds__(256) void mlp_last_kernel(const LastArgs a) {
+  constexpr int P = S_IN > 0 ? S_IN : 1;
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= a.n) return;
-  f32x4 part[kWidth / 256][S_IN];
+  f32x4 part[kWidth / 256][P];
 #pragma unroll
   for (int i = 0; i < kWidth / 256; ++i)
 #pragma unroll
-    for (int s = 0; s < S_IN; ++s)
+    for (int s = 0; s < P; ++s)
       part[i][s] = *reinterpret_cast<const f32x4*>(
           a.p_in + ((size_t)s * a.m_pad + row) * kWidth + 256 * i + 4 * lane);
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < kWidth / 256; ++i) {
     const int k = 256 * i + 4 * lane;
-    f32x4 v = *reinterpret_cast<const f32x4*>(a.bias_in + k);
+    f32x4 v = part[i][0];
+    if (S_IN > 0) {
+      v = *reinterpret_cast<const f32x4*>(a.bias_in + k);
 #pragma unroll
-    for (int s = 0; s < S_IN; ++s) v += part[i][s];
+      for (int s = 0; s < S_IN; ++s) v += part[i][s];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = fmaxf(v[e], 0.f);
+    }
     const f32x4 wl = *reinterpret_cast<const f32x4*>(a.w_last + k);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) sum = fmaf(fmaxf(v[e], 0.f), wl[e], sum);
+    for (int e = 0; e < 4; ++e) sum = fmaf(v[e], wl[e], sum);
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off);
@@ -421,7 +480,7 @@ struct hbt_mlp {
   const float* bias;
   const float* w_last;
   float b_last;
-  float* scratch[2];   // few-rows path: two buffers of [kSplit][kSmallMaxRows][width] partials
+  float* scratch[2];   // per-layer path: two buffers of kScratchFloats activations or partials
 };
 
 namespace hbt {
@@ -492,7 +551,7 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
   const size_t off_bias = off; off = align_up(off + sizeof(float) * n_bias, 256);
   const size_t off_last = off; off = align_up(off + sizeof(float) * kWidth, 256);
   const size_t image = off;  // what is copied from the host; scratch follows
-  const size_t scratch_bytes = sizeof(float) * kSplit * kSmallMaxRows * kWidth;
+  const size_t scratch_bytes = sizeof(float) * kScratchFloats;
   const size_t off_scratch0 = off; off = align_up(off + scratch_bytes, 256);
   const size_t off_scratch1 = off; off = align_up(off + scratch_bytes, 256);
   const size_t total = off;
@@ -580,51 +639,49 @@ int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* 
   if (device != mlp->device) return HBT_EINVAL;
 
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-  if (n <= kSmallMaxRows) {
-    // one launch per layer, K-partials through the handle's scratch buffers
+  if (n <= kLayerMaxRows) {
+    // one launch per layer, through the handle's two scratch buffers
     const int m_tiles = (int)((n + kRows - 1) / kRows);
-    const int groups_total = mlp->in_padded / 8 + mlp->hidden * (kWidth / 8);
+    const bool split_k = m_tiles == 1;
     LayerArgs l{};
     l.w_stream = mlp->w_stream;
-    l.groups_total = groups_total;
+    l.groups_total = mlp->in_padded / 8 + mlp->hidden * (kWidth / 8);
     l.raw = raw_features; l.mu = mlp->mu; l.sigma = mlp->sigma;
     l.in_features = mlp->in_features;
     l.n = n;
     l.m_pad = m_tiles * kRows;
-    const bool wide = m_tiles > 2;  // several n-tiles per workgroup once rows are re-read often
-    int s_in = 0;
+    bool partials = false;
     const float* p_in = nullptr;
     for (int layer = 0; layer <= mlp->hidden; ++layer) {
       l.g0 = (layer == 0) ? 0 : mlp->in_padded / 8 + (layer - 1) * (kWidth / 8);
       l.kg = (layer == 0) ? mlp->in_padded / 8 : kWidth / 8;
-      l.splits = (layer == 0) ? 1 : kSplit;
-      l.p_in = p_in; l.s_in = s_in;
+      l.splits = (layer > 0 && split_k) ? kSplit : 1;
+      l.p_in = p_in;
       l.bias_in = (layer == 0) ? nullptr : mlp->bias + (size_t)(layer - 1) * kWidth;
+      l.bias_out = mlp->bias + (size_t)layer * kWidth;
       l.p_out = mlp->scratch[layer & 1];
-      const dim3 grid(wide ? 8 : 32, (unsigned)l.splits, (unsigned)m_tiles);
-      if (layer == 0) {
-        if (wide) hipLaunchKernelGGL((mlp_layer_kernel<4, true, 1>), grid, dim3(256), 0, stream, l);
-        else hipLaunchKernelGGL((mlp_layer_kernel<1, true, 1>), grid, dim3(256), 0, stream, l);
-      } else if (s_in == 1) {
-        if (wide) hipLaunchKernelGGL((mlp_layer_kernel<4, false, 1>), grid, dim3(256), 0, stream, l);
-        else hipLaunchKernelGGL((mlp_layer_kernel<1, false, 1>), grid, dim3(256), 0, stream, l);
-      } else {
-        if (wide)
-          hipLaunchKernelGGL((mlp_layer_kernel<4, false, kSplit>), grid, dim3(256), 0, stream, l);
-        else
-          hipLaunchKernelGGL((mlp_layer_kernel<1, false, kSplit>), grid, dim3(256), 0, stream, l);
-      }
+      const dim3 grid(kWidth / 32, (unsigned)l.splits, (unsigned)m_tiles);
+      if (layer == 0)
+        hipLaunchKernelGGL((mlp_layer_kernel<true, 0, true, 4, false>), grid, dim3(256), 0, stream, l);
+      else if (!split_k)
+        hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true>), grid, dim3(512), 0, stream, l);
+      else if (partials)
+        hipLaunchKernelGGL((mlp_layer_kernel<false, kSplit, false, 4, false>), grid, dim3(256), 0,
+                           stream, l);
+      else
+        hipLaunchKernelGGL((mlp_layer_kernel<false, 0, false, 4, false>), grid, dim3(256), 0,
+                           stream, l);
       p_in = l.p_out;
-      s_in = l.splits;
+      partials = l.splits != 1;
     }
     LastArgs z{};
-    z.p_in = p_in; z.s_in = s_in;
+    z.p_in = p_in;
     z.bias_in = mlp->bias + (size_t)mlp->hidden * kWidth;
     z.w_last = mlp->w_last; z.b_last = mlp->b_last;
     z.n = n; z.m_pad = l.m_pad; z.out = out;
     const dim3 rows_grid((unsigned)((n + 3) / 4));
-    if (s_in == 1) hipLaunchKernelGGL(mlp_last_kernel<1>, rows_grid, dim3(256), 0, stream, z);
-    else hipLaunchKernelGGL(mlp_last_kernel<kSplit>, rows_grid, dim3(256), 0, stream, z);
+    if (partials) hipLaunchKernelGGL(mlp_last_kernel<kSplit>, rows_grid, dim3(256), 0, stream, z);
+    else hipLaunchKernelGGL(mlp_last_kernel<0>, rows_grid, dim3(256), 0, stream, z);
     return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
   }
 

@@ -163,10 +163,14 @@ def test_predictor_on_resnet50_shaped_trace():
         tol = 1e-4 if op.name in ("conv2d", "linear") else 1e-6
         assert g == pytest.approx(w, rel=tol), op.name
     assert predicted.run_time_ms == pytest.approx(opred.trace_ms(want), rel=1e-5)
-    # one operation at a time gives the same numbers as the batched call
+    # one operation at a time gives the same numbers as the batched call (for
+    # the MLP operations up to fp32 rounding: one row and fifty-four rows are
+    # summed over K in different orders)
     for idx in (0, 1, 5, len(trace.operations) - 1):
-        single = predictor.predict_operation(trace.operations[idx], dest)
-        assert single.run_time_ms == pytest.approx(got[idx], rel=1e-12)
+        op = trace.operations[idx]
+        single = predictor.predict_operation(op, dest)
+        tol = 1e-6 if op.name in ("conv2d", "linear") else 1e-12
+        assert single.run_time_ms == pytest.approx(got[idx], rel=tol)
     assert trace.to_device(origin, predictor) is trace
     with pytest.raises(RuntimeError):
         predicted.operations[0].to_device(origin, predictor)
