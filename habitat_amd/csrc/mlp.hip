@@ -248,8 +248,8 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
 // 33.6 MB of weights through by itself (about 1 ms), and any batch below 8192
 // rows leaves compute units idle for that long.  Here a layer is spread over
 // the chip instead: a workgroup takes one n-tile x one m-tile, its waves split
-// K, each issues the loads of all its k-groups at once, multiplies them as
-// they arrive and the waves add their 32 x 32 accumulators through LDS.
+// K, each multiplies its k-groups straight from global memory (no loop, no LDS
+// staging) and the waves add their 32 x 32 accumulators through LDS.
 //
 //   33 rows and more: eight waves cover all of K (16 k-groups each), the
 //   workgroup applies bias and ReLU and writes activations, [row][n].
@@ -263,6 +263,7 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
 // weights, same MFMA instruction, same fragment layout as above.
 constexpr int kSplit = 8;            // K-partials per hidden layer, up to kRows rows
 constexpr int kLayerMaxRows = 4096;  // largest batch that takes this path
+constexpr int kFewTiles = 8;         // m-tiles up to which the whole-K shape prefetches (DEPTH)
 constexpr size_t kScratchFloats = (size_t)kLayerMaxRows * kWidth;  // each of two buffers
 static_assert((size_t)kSplit * kRows * kWidth <= kScratchFloats, "the K-partials fit the scratch");
 
@@ -307,7 +308,13 @@ struct LayerFrag {
 //     padded m-tile holds them) instead of being masked; masking saves most of
 //     the traffic of a handful of rows, not masking keeps the loads of a full
 //     tile free of branches.
-template <bool FIRST, int S_IN, bool FINAL, int WAVES, bool PADDED_ROWS>
+//   DEPTH: k-groups whose loads are kept in flight ahead of the MFMAs; 0 leaves
+//     the placement to the compiler.  Measured for the whole-K shape (us per
+//     forward at 64 / 256 / 512 / 4096 rows): 0: 80 88 132 766; 2: 70 77 137
+//     841; 4: 76 83 154 1014; 8: 90 97 188 1338; all 16: 95 102 178 1199.  More
+//     loads in flight only crowd the path from L2 once every compute unit has
+//     several workgroups; with a few m-tiles two groups ahead is best.
+template <bool FIRST, int S_IN, bool FINAL, int WAVES, bool PADDED_ROWS, int DEPTH>
 __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a) {
   static_assert(S_IN == 0 || !FINAL, "K-partials go in and come out together");
   static_assert(WAVES == 4 || WAVES == 8, "the reduction below is written for these");
@@ -336,11 +343,9 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
                         ((size_t)(tile >> 3) * a.groups_total + a.g0) * (8 * 64) +
                         (tile & 7) * 64 + lane;
 
-  // every load of the wave, then the arithmetic in the order of arrival
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   LayerFrag<G, S_IN> f;
-#pragma unroll
-  for (int j = 0; j < G; ++j) {
+  auto load_group = [&](int j) {
     if (!FIRST || j < count) {
       const int gl = first + j;  // layer-local group
       f.w[j] = w_lane[(size_t)gl * (8 * 64)];
@@ -368,13 +373,12 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
         f.bias[j] = *reinterpret_cast<const f32x4*>(a.bias_in + k);
       }
     }
-  }
+  };
 
   f32x16 acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-#pragma unroll
-  for (int j = 0; j < G; ++j) {
+  auto mfma_group = [&](int j) {
     if (!FIRST || j < count) {
       f32x4 v = f.x[j][0];
       if (S_IN > 0) {
@@ -388,6 +392,26 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(f.w[j][e], v[e], acc, 0, 0, 0);
+    }
+  };
+
+  if (DEPTH == 0) {
+    // the compiler places the loads: each group's next to its MFMAs, one trip
+    // to memory after the other, which resident workgroups hide from each other
+#pragma unroll
+    for (int j = 0; j < G; ++j) load_group(j);
+#pragma unroll
+    for (int j = 0; j < G; ++j) mfma_group(j);
+  } else {
+    // DEPTH groups in flight ahead of the MFMAs
+#pragma unroll
+    for (int j = 0; j < (DEPTH < G ? DEPTH : G); ++j) load_group(j);
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+      if (j + DEPTH < G) load_group(j + DEPTH);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_group(j);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
@@ -662,14 +686,19 @@ int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* 
       l.p_out = mlp->scratch[layer & 1];
       const dim3 grid(kWidth / 32, (unsigned)l.splits, (unsigned)m_tiles);
       if (layer == 0)
-        hipLaunchKernelGGL((mlp_layer_kernel<true, 0, true, 4, false>), grid, dim3(256), 0, stream, l);
-      else if (!split_k)
-        hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true>), grid, dim3(512), 0, stream, l);
-      else if (partials)
-        hipLaunchKernelGGL((mlp_layer_kernel<false, kSplit, false, 4, false>), grid, dim3(256), 0,
+        hipLaunchKernelGGL((mlp_layer_kernel<true, 0, true, 4, false, 0>), grid, dim3(256), 0,
                            stream, l);
+      else if (!split_k && m_tiles <= kFewTiles)
+        hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 2>), grid, dim3(512), 0,
+                           stream, l);
+      else if (!split_k)
+        hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 0>), grid, dim3(512), 0,
+                           stream, l);
+      else if (partials)
+        hipLaunchKernelGGL((mlp_layer_kernel<false, kSplit, false, 4, false, 0>), grid, dim3(256),
+                           0, stream, l);
       else
-        hipLaunchKernelGGL((mlp_layer_kernel<false, 0, false, 4, false>), grid, dim3(256), 0,
+        hipLaunchKernelGGL((mlp_layer_kernel<false, 0, false, 4, false, 0>), grid, dim3(256), 0,
                            stream, l);
       p_in = l.p_out;
       partials = l.splits != 1;
