@@ -119,7 +119,7 @@ int hbt_occupancy_host_model32_batch(const hbt_device_spec* spec, int64_t n,
   if (!d.fast_ok()) return HBT_ESPEC;
   // the form the kernels run for this device: the straight-line one where the
   // device allows it
-  const bool lean = d.lean_ok(), cdna_lean = d.cdna_lean_ok();
+  const bool lean = d.lean_ok(), lean_gp = d.lean_gp_ok(), cdna_lean = d.cdna_lean_ok();
   for (int64_t i = 0; i < n; ++i) {
     const int32_t smem_total = hbt::smem_sum(static_smem[i], dynamic_smem[i]);
     const int32_t r = regs[i] & 0xFFFF;
@@ -128,8 +128,9 @@ int hbt_occupancy_host_model32_batch(const hbt_device_spec* spec, int64_t n,
       out[i] = cdna_lean ? hbt::occupancy_cdna<false, true>(d, b, smem_total, r)
                          : hbt::occupancy_cdna<false>(d, b, smem_total, r);
     else
-      out[i] = lean ? hbt::occupancy_fast<true>(d, b, hbt::smem_alloc(smem_total), r)
-                    : hbt::occupancy_fast<false>(d, b, hbt::smem_alloc(smem_total), r);
+      out[i] = lean      ? hbt::occupancy_fast<true>(d, b, hbt::smem_alloc(smem_total), r)
+               : lean_gp ? hbt::occupancy_fast<true, true>(d, b, hbt::smem_alloc(smem_total), r)
+                         : hbt::occupancy_fast<false>(d, b, hbt::smem_alloc(smem_total), r);
   }
   return HBT_OK;
 }

@@ -80,6 +80,12 @@ struct OccDevice {
     return (flags & (kOk | kFastOk | kWarpPow2 | kCdna | kGp100 | kPoolSteps)) ==
            (kOk | kFastOk | kWarpPow2);
   }
+  // lean_ok, or that but for the cc 6.0 re-check (the P100), which the kernels
+  // then apply by a select on the flag instead of a branch
+  HBT_HD bool lean_gp_ok() const {
+    return (flags & (kOk | kFastOk | kWarpPow2 | kCdna | kPoolSteps)) ==
+           (kOk | kFastOk | kWarpPow2);
+  }
   // likewise for the compute-unit model: an accepted AMD description with
   // small limits and a power-of-two wavefront size
   HBT_HD bool cdna_lean_ok() const {
@@ -232,9 +238,10 @@ HBT_HD SmemAlloc smem_alloc(int32_t smem_total) {
 // monotonic, so min(floor(a / w), floor(b / w)) is taken as floor(min(a, b) / w).
 //
 // LEAN: the device has lean_ok(), so none of the wave-uniform branches is
-// compiled in and the whole model is one basic block (the kernel then
-// interleaves the arithmetic of a thread's records).
-template <bool LEAN = false>
+// compiled in and the whole model is one basic block.  GP_SELECT (with LEAN):
+// the device has lean_gp_ok(); the cc 6.0 re-check is computed for every
+// record and applied where the device's flag says so, still without a branch.
+template <bool LEAN = false, bool GP_SELECT = false>
 HBT_HD int32_t occupancy_fast(const OccDevice& d, int32_t block, const SmemAlloc& sm,
                               int32_t regs) {
   if (!LEAN && !d.ok()) return 0;
@@ -262,12 +269,13 @@ HBT_HD int32_t occupancy_fast(const OccDevice& d, int32_t block, const SmemAlloc
   const int32_t per_warp1 = per_warp > 0 ? per_warp : 1;
   const float rcp_per_warp = fast_rcp(per_warp1);
   const int32_t reg_warps = fast_div_r(d.regs_per_subpart, per_warp1, rcp_per_warp) << d.sub_shift;
-  if (!LEAN && (d.flags & kGp100)) {
+  if (GP_SELECT || (!LEAN && (d.flags & kGp100))) {
     // cc 6.0 must also fit a 4-sub-partition Pascal SM
     const int32_t warps_up4 = (warps + 3) & ~3;
-    fits = fits && mul_small(per_warp256, warps_up4) <= block_regs256 &&
-           (per_warp == 0 ||
-            (fast_div_r(d.regs_per_subpart4, per_warp1, rcp_per_warp) << 2) >= warps);
+    const bool fits4 = mul_small(per_warp256, warps_up4) <= block_regs256 &&
+                       (per_warp == 0 ||
+                        (fast_div_r(d.regs_per_subpart4, per_warp1, rcp_per_warp) << 2) >= warps);
+    fits = fits && (fits4 || (GP_SELECT && !(d.flags & kGp100)));
   }
   int32_t warp_budget = d.max_warps_per_sm;
   warp_budget = (per_warp > 0 && reg_warps < warp_budget) ? reg_warps : warp_budget;

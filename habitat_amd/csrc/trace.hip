@@ -232,14 +232,9 @@ hbt_device_table* hbt_device_table_create(const hbt_device_spec* origin,
   t->n_dest = n_dest;
   t->device = device;
   t->origin = make_origin_args(*origin);
-  bool lean = true, cdna = true;
   std::vector<DestArgs> host((size_t)n_dest);
-  for (int32_t d = 0; d < n_dest; ++d) {
-    host[d] = make_dest_args(*origin, dests[d]);
-    lean = lean && host[d].dev.lean_ok();
-    cdna = cdna && host[d].dev.cdna_lean_ok();
-  }
-  t->model = dev::model_for(t->origin.dev.lean_ok(), t->origin.dev.cdna_lean_ok(), lean, cdna);
+  for (int32_t d = 0; d < n_dest; ++d) host[d] = make_dest_args(*origin, dests[d]);
+  t->model = dev::model_for(t->origin.dev, host.data(), n_dest);
   t->dests = nullptr;
   const size_t bytes = sizeof(DestArgs) * (size_t)n_dest;
   if (hipMalloc(reinterpret_cast<void**>(&t->dests), bytes) != hipSuccess) {

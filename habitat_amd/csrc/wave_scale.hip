@@ -220,13 +220,7 @@ void launch(const WaveScaleArgs& args, hipStream_t stream) {
 
 hipError_t launch_wave_scale(const WaveScaleArgs& args, bool vectorised, hipStream_t stream) {
   if (args.n <= 0) return hipSuccess;
-  bool lean = true, cdna = true;
-  for (int d = 0; d < args.n_dest; ++d) {
-    lean = lean && args.dest[d].dev.lean_ok();
-    cdna = cdna && args.dest[d].dev.cdna_lean_ok();
-  }
-  const int model =
-      model_for(args.origin.dev.lean_ok(), args.origin.dev.cdna_lean_ok(), lean, cdna);
+  const int model = model_for(args.origin.dev, args.dest, args.n_dest);
   const bool vec = vectorised && kRecPerThread > 1;
   with_model(model, [&](auto m) {
     if (vec) launch<kRecPerThread, decltype(m)::value>(args, stream);

@@ -100,11 +100,13 @@ struct C100 { static constexpr double value = 100.0; };
 struct C1e9 { static constexpr double value = 1e9; };
 
 // Which occupancy models a kernel instantiation contains.
-//   The four lean ones: the origin and every destination of the launch have
+//   The lean ones: the origin and every destination of the launch have
 //     OccDevice::lean_ok (the 32-bit NVIDIA-rule model, straight-line) or
 //     cdna_lean_ok (the compute-unit model, straight-line), the origin one kind
 //     and the destinations all one kind; nothing else is compiled in and no
-//     branch is uniform over the launch.
+//     branch is uniform over the launch.  kModelLeanGp: NVIDIA-rule devices
+//     with a P100 among them (lean_gp_ok): the cc 6.0 re-check is computed for
+//     every record and selected by the device's flag.
 //   kModelGeneral: each device picks its model by wave-uniform branches: the
 //     compute-unit model for AMD descriptions, the 64-bit model with real
 //     divisions for devices with limits of 2^20 and more (not real hardware,
@@ -115,16 +117,22 @@ enum : int {
   kModelLeanCdnaDest = 2,    // NVIDIA-rule origin, AMD destinations
   kModelLeanCdnaOrigin = 3,  // AMD origin, NVIDIA-rule destinations
   kModelLeanCdna = 4,        // AMD origin and destinations
+  kModelLeanGp = 5,          // NVIDIA-rule origin and destinations, cc 6.0 among them
 };
 
-// The instantiation for a launch whose origin and destinations are of these
-// kinds (each: lean_ok, cdna_lean_ok, or neither).
-inline int model_for(bool origin_lean, bool origin_cdna_lean, bool dests_lean,
-                     bool dests_cdna_lean) {
-  if (origin_lean && dests_lean) return kModelLean;
-  if (origin_lean && dests_cdna_lean) return kModelLeanCdnaDest;
-  if (origin_cdna_lean && dests_lean) return kModelLeanCdnaOrigin;
-  if (origin_cdna_lean && dests_cdna_lean) return kModelLeanCdna;
+// The instantiation for a launch from `origin` to the n_dest devices of `dests`.
+inline int model_for(const OccDevice& origin, const DestArgs* dests, int n_dest) {
+  bool lean = true, gp = true, cdna = true;
+  for (int d = 0; d < n_dest; ++d) {
+    lean = lean && dests[d].dev.lean_ok();
+    gp = gp && dests[d].dev.lean_gp_ok();
+    cdna = cdna && dests[d].dev.cdna_lean_ok();
+  }
+  if (origin.lean_ok() && lean) return kModelLean;
+  if (origin.lean_ok() && cdna) return kModelLeanCdnaDest;
+  if (origin.cdna_lean_ok() && lean) return kModelLeanCdnaOrigin;
+  if (origin.cdna_lean_ok() && cdna) return kModelLeanCdna;
+  if (origin.lean_gp_ok() && gp) return kModelLeanGp;
   return kModelGeneral;
 }
 
@@ -136,6 +144,7 @@ inline void with_model(int model, F&& f) {
     case kModelLeanCdnaDest: f(std::integral_constant<int, kModelLeanCdnaDest>()); break;
     case kModelLeanCdnaOrigin: f(std::integral_constant<int, kModelLeanCdnaOrigin>()); break;
     case kModelLeanCdna: f(std::integral_constant<int, kModelLeanCdna>()); break;
+    case kModelLeanGp: f(std::integral_constant<int, kModelLeanGp>()); break;
     default: f(std::integral_constant<int, kModelGeneral>()); break;
   }
 }
@@ -148,6 +157,7 @@ __device__ __forceinline__ int32_t occupancy_dev(const OccDevice& d, int32_t blo
   constexpr bool cdna = DEST ? (MODEL == kModelLeanCdnaDest || MODEL == kModelLeanCdna)
                              : (MODEL == kModelLeanCdnaOrigin || MODEL == kModelLeanCdna);
   if (cdna) return occupancy_cdna<false, true>(d, block, smem_total, regs);
+  if (MODEL == kModelLeanGp) return occupancy_fast<true, true>(d, block, sm, regs);
   if (MODEL != kModelGeneral) return occupancy_fast<true>(d, block, sm, regs);
   if (d.flags & kCdna)
     return d.fast_ok() ? occupancy_cdna<false>(d, block, smem_total, regs)

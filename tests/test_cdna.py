@@ -184,14 +184,16 @@ def test_strategy_and_sweep_use_the_compute_unit_model():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("case", ["nvidia_to_amd", "amd_to_nvidia", "amd_to_amd"])
+@pytest.mark.parametrize("case", ["nvidia_to_amd", "amd_to_nvidia", "amd_to_amd", "with_p100",
+                                  "from_p100"])
 def test_lean_and_general_instantiations_agree_bit_for_bit(case):
-    """A launch whose origin and destinations are each of one kind (NVIDIA-rule
-    or AMD description) runs a kernel instantiation without the model's uniform
-    branches; a P100 among the destinations forces the general one.  Same
-    records, same first destination: every output of that destination must be
-    identical, on ordinary records and on field values at and beyond the limits,
-    and the occupancies must be the host routine's."""
+    """A launch whose origin and destinations are each of one kind (NVIDIA-rule,
+    with or without a P100 among them, or AMD description) runs a kernel
+    instantiation without the model's uniform branches; destinations of mixed
+    kinds force the general one.  Same records, same first destination: every
+    output of that destination must be identical, on ordinary records and on
+    field values at and beyond the limits, and the occupancies must be the host
+    routine's."""
     import torch
     from test_wave_scale_gpu import adversarial_records
     from habitat_amd import DeviceProperties
@@ -203,14 +205,16 @@ def test_lean_and_general_instantiations_agree_bit_for_bit(case):
         amd.as_dict(), compute_minor=2, shared_mem_per_block=65536,
         shared_mem_per_multiprocessor=65536, num_sms=304, mem_bandwidth_gb=5300,
         base_clock_mhz=2100, peak_gflops_per_second=163400))
-    origin, first, other = {"nvidia_to_amd": (Device.V100, amd, amd2),
-                            "amd_to_nvidia": (amd, Device.V100, Device.T4),
-                            "amd_to_amd": (amd2, amd, amd2)}[case]
+    origin, first, other, mixer = {"nvidia_to_amd": (Device.V100, amd, amd2, Device.P100),
+                                   "amd_to_nvidia": (amd, Device.V100, Device.T4, Device.P100),
+                                   "amd_to_amd": (amd2, amd, amd2, Device.P100),
+                                   "with_p100": (Device.V100, Device.P100, Device.T4, amd),
+                                   "from_p100": (Device.P100, Device.V100, Device.P100, amd)}[case]
     ordinary, _ = synthetic.kernel_records(50_001, Device.V100, seed=5, metrics_fraction=0.8)
     for rec in (ordinary, adversarial_records(40_003, 17)):
         kr = KernelRecords.from_numpy(rec)
         lean = wave_scale(kr, origin, [first, other], waves=True)
-        general = wave_scale(kr, origin, [first, Device.P100], waves=True)
+        general = wave_scale(kr, origin, [first, mixer], waves=True)
         single = wave_scale(kr, origin, [first], waves=True)
         for out in (lean, single):
             for name in ("time_ns", "occ_dest", "wave_dest", "status"):
@@ -229,7 +233,7 @@ def test_lean_and_general_instantiations_agree_bit_for_bit(case):
         seg = torch.arange(kr.n, dtype=torch.int32, device=kr.device) // 1000
         n_seg = (kr.n + 999) // 1000
         sums_lean, bad_lean = wave_scale_sum(kr, DeviceTable(origin, [first, other]), seg, n_seg)
-        sums_gen, bad_gen = wave_scale_sum(kr, DeviceTable(origin, [first, Device.P100]), seg,
+        sums_gen, bad_gen = wave_scale_sum(kr, DeviceTable(origin, [first, mixer]), seg,
                                            n_seg)
         assert torch.equal(bad_lean[0], bad_gen[0])
         a, b = sums_lean[0].cpu().numpy(), sums_gen[0].cpu().numpy()
