@@ -124,7 +124,7 @@ def tile_records(rec, n):
 
 def mlp_bench(args):
     """configs[2] (and the other kinds of configs[3], one step each): the fused
-    MLP at full size, the few-rows path, and a torch CPU baseline."""
+    MLP at full size, the per-layer path (up to 4096 rows), and a torch CPU baseline."""
     import torch
     from habitat_amd import synthetic
     from habitat_amd.analysis.mlp.mlp import RuntimePredictor

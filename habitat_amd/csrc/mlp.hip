@@ -451,7 +451,7 @@ struct LastArgs {
   float* out;            // [n]
 };
 
-// fc2 for few rows: one wavefront per row.  S_IN as in mlp_layer_kernel.
+// fc2 after the per-layer kernels: one wavefront per row.  S_IN as in mlp_layer_kernel.
 template <int S_IN>
 __global__ __launch_bounds__(256) void mlp_last_kernel(const LastArgs a) {
   constexpr int P = S_IN > 0 ? S_IN : 1;
