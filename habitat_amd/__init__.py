@@ -46,7 +46,7 @@ _SUBMODULES = [
     "analysis.wave_scaling", "analysis.wave_scaling.common", "analysis.wave_scaling.metadata",
     "analysis.wave_scaling.resimplified", "analysis.wave_scaling.roofline",
     "analysis.wave_scaling.unified", "analysis.wave_scaling.batch", "analysis.wave_scaling.cdna",
-    "analysis.report", "analysis.sweep", "data", "device",
+    "analysis.report", "analysis.sweep", "data", "device", "utils",
 ]
 
 

@@ -211,7 +211,10 @@ def test_habitat_alias_imports():
     from habitat.analysis.device import _Device  # noqa: F401
     from habitat.analysis.wave_scaling.roofline import _ridge_point
     from habitat.analysis.trace import Trace  # noqa: F401  (no data files needed to import)
+    from habitat.utils import ms_to_ns, name_all_arguments, ns_to_ms
     import habitat
+    assert ns_to_ms(ms_to_ns(2.5)) == 2.5
+    assert name_all_arguments(["a", "b", "c"], (1, 2), {"c": 3}) == {"a": 1, "b": 2, "c": 3}
     assert _ridge_point(habitat.Device.T4) == 1804 / 239
     assert habitat.Device.V100.num_sms == 80
     k = KernelInstance("k", 4096, 256, 0, 0, 32, 1000000)
