@@ -12,7 +12,8 @@ inputs resident in HBM.  Prints ONE JSON line:
                 launch stream)
   cpu_baseline  the CPU oracle (C restatement of the reference's per-kernel
                 Python, one thread) on the same records, same machine
-  large         the same kernel at 64 M records (beyond the 256 MB last-level cache)
+  large         the same kernel at 64 M records (beyond the 256 MB last-level cache);
+                large_16M: at 16 M records
   mlp           the fused MFMA MLP (configs[2], conv2d, 1 M rows): rows/s, its
                 roofline against fp32 MFMA peak and a torch-CPU fp32 baseline
   sweep         configs[4]: one ResNet-50-shaped trace predicted for 256 devices
@@ -413,8 +414,8 @@ def main():
         attempt("cpu_baseline", cpu_section)
 
     # ---------------- the same kernel beyond the last-level cache ----------------
-    def large_section():
-        big = KernelRecords.from_numpy(tile_records(rec, args.large_records))
+    def large_section(n_records=None):
+        big = KernelRecords.from_numpy(tile_records(rec, n_records or args.large_records))
         big_out = WaveScaleOutput(big.n, 1, big.device, waves=False, status=True)
         big_call = WaveScaleCall(big, origin, dest, big_out)
         steps = max(5, min(args.steps, 40))
@@ -430,6 +431,10 @@ def main():
     if not args.no_large and args.large_records > args.records:
         attempt("large", large_section)
         torch.cuda.empty_cache()
+        # a size between the two: out of L2, within the last-level cache's reach
+        if args.large_records > 16_000_000 > args.records:
+            attempt("large_16M", lambda: large_section(16_000_000))
+            torch.cuda.empty_cache()
 
     # ---------------- MLP, configs[2] ----------------
     if not args.no_mlp:
