@@ -497,6 +497,7 @@ constexpr size_t kLdsBytes =
 struct hbt_mlp {
   int32_t in_features, in_padded, width, hidden;
   int device;
+  int compute_units;   // of that device: the fused kernel runs one workgroup on each
   void* blob;          // one device allocation holding everything below
   const double* mu;
   const double* sigma;
@@ -533,6 +534,88 @@ size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 }  // namespace
 }  // namespace hbt
 
+namespace {
+
+// One launch per layer for n <= kLayerMaxRows rows, through the handle's two
+// scratch buffers.
+int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* out,
+                   hipStream_t stream) {
+  using namespace hbt;
+  // one launch per layer, through the handle's two scratch buffers
+  const int m_tiles = (int)((n + kRows - 1) / kRows);
+  const bool split_k = m_tiles == 1;
+  LayerArgs l{};
+  l.w_stream = mlp->w_stream;
+  l.groups_total = mlp->in_padded / 8 + mlp->hidden * (kWidth / 8);
+  l.raw = raw_features; l.mu = mlp->mu; l.sigma = mlp->sigma;
+  l.in_features = mlp->in_features;
+  l.n = n;
+  l.m_pad = m_tiles * kRows;
+  bool partials = false;
+  const float* p_in = nullptr;
+  for (int layer = 0; layer <= mlp->hidden; ++layer) {
+    l.g0 = (layer == 0) ? 0 : mlp->in_padded / 8 + (layer - 1) * (kWidth / 8);
+    l.kg = (layer == 0) ? mlp->in_padded / 8 : kWidth / 8;
+    l.splits = (layer > 0 && split_k) ? kSplit : 1;
+    l.p_in = p_in;
+    l.bias_in = (layer == 0) ? nullptr : mlp->bias + (size_t)(layer - 1) * kWidth;
+    l.bias_out = mlp->bias + (size_t)layer * kWidth;
+    l.p_out = mlp->scratch[layer & 1];
+    const dim3 grid(kWidth / 32, (unsigned)l.splits, (unsigned)m_tiles);
+    if (layer == 0)
+      hipLaunchKernelGGL((mlp_layer_kernel<true, 0, true, 4, false, 0>), grid, dim3(256), 0,
+                         stream, l);
+    else if (!split_k && m_tiles <= kFewTiles)
+      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 2>), grid, dim3(512), 0,
+                         stream, l);
+    else if (!split_k)
+      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 0>), grid, dim3(512), 0,
+                         stream, l);
+    else if (partials)
+      hipLaunchKernelGGL((mlp_layer_kernel<false, kSplit, false, 4, false, 0>), grid, dim3(256),
+                         0, stream, l);
+    else
+      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, false, 4, false, 0>), grid, dim3(256), 0,
+                         stream, l);
+    p_in = l.p_out;
+    partials = l.splits != 1;
+  }
+  LastArgs z{};
+  z.p_in = p_in;
+  z.bias_in = mlp->bias + (size_t)mlp->hidden * kWidth;
+  z.w_last = mlp->w_last; z.b_last = mlp->b_last;
+  z.n = n; z.m_pad = l.m_pad; z.out = out;
+  const dim3 rows_grid((unsigned)((n + 3) / 4));
+  if (partials) hipLaunchKernelGGL(mlp_last_kernel<kSplit>, rows_grid, dim3(256), 0, stream, z);
+  else hipLaunchKernelGGL(mlp_last_kernel<0>, rows_grid, dim3(256), 0, stream, z);
+  return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
+}
+
+// The fused kernel: one workgroup per 32 rows.
+int forward_fused(hbt_mlp* mlp, const double* raw_features, int64_t n, float* out,
+                  hipStream_t stream) {
+  using namespace hbt;
+  const int64_t blocks = (n + kRows - 1) / kRows;
+  MlpArgs a{};
+  a.raw = raw_features;
+  a.out = out;
+  a.n = n;
+  a.in_features = mlp->in_features;
+  a.in_padded = mlp->in_padded;
+  a.hidden = mlp->hidden;
+  a.mu = mlp->mu;
+  a.sigma = mlp->sigma;
+  a.w_stream = mlp->w_stream;
+  a.bias = mlp->bias;
+  a.w_last = mlp->w_last;
+  a.b_last = mlp->b_last;
+  hipLaunchKernelGGL(mlp_fused_kernel<kWaves>, dim3((unsigned)blocks), dim3(kWaves * 64),
+                     kLdsBytes, stream, a);
+  return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
+}
+
+}  // namespace
+
 extern "C" {
 
 hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layers,
@@ -556,6 +639,15 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
   }
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    *err = HBT_EHIP;
+    return nullptr;
+  }
+
+  int compute_units = 0;
+  if (hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device) !=
+          hipSuccess ||
+      compute_units <= 0) {
     (void)hipGetLastError();
     *err = HBT_EHIP;
     return nullptr;
@@ -632,6 +724,7 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
   m->width = width;
   m->hidden = hidden_layers;
   m->device = device;
+  m->compute_units = compute_units;
   m->blob = blob;
   m->mu = reinterpret_cast<const double*>(base + off_mu);
   m->sigma = reinterpret_cast<const double*>(base + off_sigma);
@@ -663,73 +756,19 @@ int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* 
   if (device != mlp->device) return HBT_EINVAL;
 
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-  if (n <= kLayerMaxRows) {
-    // one launch per layer, through the handle's two scratch buffers
-    const int m_tiles = (int)((n + kRows - 1) / kRows);
-    const bool split_k = m_tiles == 1;
-    LayerArgs l{};
-    l.w_stream = mlp->w_stream;
-    l.groups_total = mlp->in_padded / 8 + mlp->hidden * (kWidth / 8);
-    l.raw = raw_features; l.mu = mlp->mu; l.sigma = mlp->sigma;
-    l.in_features = mlp->in_features;
-    l.n = n;
-    l.m_pad = m_tiles * kRows;
-    bool partials = false;
-    const float* p_in = nullptr;
-    for (int layer = 0; layer <= mlp->hidden; ++layer) {
-      l.g0 = (layer == 0) ? 0 : mlp->in_padded / 8 + (layer - 1) * (kWidth / 8);
-      l.kg = (layer == 0) ? mlp->in_padded / 8 : kWidth / 8;
-      l.splits = (layer > 0 && split_k) ? kSplit : 1;
-      l.p_in = p_in;
-      l.bias_in = (layer == 0) ? nullptr : mlp->bias + (size_t)(layer - 1) * kWidth;
-      l.bias_out = mlp->bias + (size_t)layer * kWidth;
-      l.p_out = mlp->scratch[layer & 1];
-      const dim3 grid(kWidth / 32, (unsigned)l.splits, (unsigned)m_tiles);
-      if (layer == 0)
-        hipLaunchKernelGGL((mlp_layer_kernel<true, 0, true, 4, false, 0>), grid, dim3(256), 0,
-                           stream, l);
-      else if (!split_k && m_tiles <= kFewTiles)
-        hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 2>), grid, dim3(512), 0,
-                           stream, l);
-      else if (!split_k)
-        hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 0>), grid, dim3(512), 0,
-                           stream, l);
-      else if (partials)
-        hipLaunchKernelGGL((mlp_layer_kernel<false, kSplit, false, 4, false, 0>), grid, dim3(256),
-                           0, stream, l);
-      else
-        hipLaunchKernelGGL((mlp_layer_kernel<false, 0, false, 4, false, 0>), grid, dim3(256), 0,
-                           stream, l);
-      p_in = l.p_out;
-      partials = l.splits != 1;
-    }
-    LastArgs z{};
-    z.p_in = p_in;
-    z.bias_in = mlp->bias + (size_t)mlp->hidden * kWidth;
-    z.w_last = mlp->w_last; z.b_last = mlp->b_last;
-    z.n = n; z.m_pad = l.m_pad; z.out = out;
-    const dim3 rows_grid((unsigned)((n + 3) / 4));
-    if (partials) hipLaunchKernelGGL(mlp_last_kernel<kSplit>, rows_grid, dim3(256), 0, stream, z);
-    else hipLaunchKernelGGL(mlp_last_kernel<0>, rows_grid, dim3(256), 0, stream, z);
-    return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
-  }
-
-  MlpArgs a{};
-  a.raw = raw_features;
-  a.out = out;
-  a.n = n;
-  a.in_features = mlp->in_features;
-  a.in_padded = mlp->in_padded;
-  a.hidden = mlp->hidden;
-  a.mu = mlp->mu;
-  a.sigma = mlp->sigma;
-  a.w_stream = mlp->w_stream;
-  a.bias = mlp->bias;
-  a.w_last = mlp->w_last;
-  a.b_last = mlp->b_last;
-  hipLaunchKernelGGL(mlp_fused_kernel<kWaves>, dim3((unsigned)blocks), dim3(kWaves * 64),
-                     kLdsBytes, stream, a);
-  return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
+  if (n <= kLayerMaxRows) return forward_layers(mlp, raw_features, n, out, stream);
+  // The fused kernel keeps every compute unit busy for whole rounds of
+  // 32 rows x compute units (about 1 ms each); what is left over after the last
+  // whole round would cost another one.  Up to kLayerMaxRows leftover rows go
+  // through the per-layer path instead, which takes less.
+  const int64_t round_rows = (int64_t)kRows * mlp->compute_units;
+  const int64_t leftover = n % round_rows;
+  if (leftover == 0 || leftover > kLayerMaxRows)
+    return forward_fused(mlp, raw_features, n, out, stream);
+  const int64_t whole = n - leftover;
+  const int rc = forward_fused(mlp, raw_features, whole, out, stream);
+  if (rc != HBT_OK) return rc;
+  return forward_layers(mlp, raw_features + whole * mlp->in_features, leftover, out + whole, stream);
 }
 
 void hbt_mlp_destroy(hbt_mlp* mlp) {

@@ -77,12 +77,14 @@ def test_trained_like_weights_with_wide_output_range():
 
 
 # up to 4096 rows run one launch per layer (K split over workgroups up to 32
-# rows, whole K per workgroup above), more rows the fused kernel
+# rows, whole K per workgroup above), more rows the fused kernel in whole rounds
+# of 32 rows x 256 compute units, and up to 4096 rows left over after the last
+# whole round one launch per layer again
 @pytest.mark.parametrize("n", [1, 2, 31, 32, 33, 63, 64, 65, 96, 97, 511, 512, 513, 1000, 4095,
-                               4096, 4097, 5000])
+                               4096, 4097, 5000, 8191, 8192, 8193, 8192 + 4096, 8192 + 4097])
 def test_ragged_row_counts(n):
     rp = make("lstm")
-    x, mu, sigma = synthetic.mlp_features("lstm", 5000, seed=5)
+    x, mu, sigma = synthetic.mlp_features("lstm", 8192 + 4097, seed=5)
     rp.set_normalization(mu, sigma)
     y = rp.predict_batch(x[:n]).cpu().numpy()
     assert y.shape == (n,)
@@ -261,5 +263,14 @@ def test_config2_and_config3_full_size_properties(kind):
     assert_close(y.cpu().numpy()[idx], omlp.forward_fp64(rp.model.state_dict(), x[idx], mu, sigma))
     perm = torch.randperm(n, device="cuda", generator=torch.Generator("cuda").manual_seed(1))
     y_perm = rp.predict_batch(xg[perm].contiguous())
-    assert torch.equal(y_perm, y[perm])          # a row's result does not depend on its neighbours
+    # a row's result does not depend on its neighbours: bit for bit where the
+    # row is in the fused kernel's whole rounds (32 rows x 256 compute units)
+    # both times, to rounding where it is among the rows left over, which take
+    # one launch per layer
+    whole = n - n % 8192
+    pos = torch.arange(n, device="cuda")
+    fused_both = (pos < whole) & (perm < whole)
+    assert whole == 999_424 and int(fused_both.sum()) > 990_000
+    assert torch.equal(y_perm[fused_both], y[perm][fused_both])
+    assert torch.allclose(y_perm, y[perm], rtol=1e-5, atol=1e-7)
     assert bool(torch.all(torch.isfinite(y)))
