@@ -240,7 +240,7 @@ class Predictor:
                                        mode)
                 res = wave_scale(rec, occupancy_device(origin, mode),
                                  [occupancy_device(dest_device, mode)], waves=False)
-                t = res.time_ns[0].cpu().numpy()
+                t = res.time_ns[0].cpu().tolist()
                 st = res.status[0].cpu().numpy()
                 bad = np.flatnonzero(st)
                 if bad.size:
@@ -248,11 +248,9 @@ class Predictor:
             pos = 0
             for idx in idxs:
                 ks = run_times[idx].kernels
-                vals = []
-                for j, k in enumerate(ks):
-                    v = float(t[pos + j])
-                    vals.append(k.run_time_ns if v == k.run_time_ns else v)
-                times[idx] = vals
+                # an unchanged time keeps the measured value's own type (an int)
+                times[idx] = [k.run_time_ns if v == k.run_time_ns else v
+                              for k, v in zip(ks, t[pos:pos + len(ks)])]
                 pos += len(ks)
         for rt, vals in zip(run_times, times):
             preds = [PredictedKernel(k, v) for k, v in zip(rt.kernels, vals)]
