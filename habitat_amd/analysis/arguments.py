@@ -1,26 +1,24 @@
-"""Shapes and scalars an operation was called with
+"""What an operation was called with, reduced to shapes and scalars
 (analyzer/habitat/analysis/arguments.py:4-38)."""
 import torch
 
 
+def _describe(value):
+    """A tensor becomes its size; tuples and lists are walked (and come back as
+    plain tuples and lists); anything else is kept."""
+    if isinstance(value, torch.Tensor):
+        return value.size()
+    for container in (tuple, list):
+        if isinstance(value, container):
+            return container(_describe(item) for item in value)
+    return value
+
+
 class Arguments:
     def __init__(self, args, kwargs):
-        self.args = args
-        self.kwargs = kwargs
+        self.args, self.kwargs = args, kwargs
         self.special = {}
 
     @classmethod
     def from_raw_arguments(cls, args, kwargs):
-        return cls(tuple(_shape_of(a) for a in args),
-                   {name: _shape_of(value) for name, value in kwargs.items()})
-
-
-def _shape_of(argument):
-    """Tensors are replaced by their sizes; containers are walked; scalars stay."""
-    if isinstance(argument, tuple):
-        return tuple(_shape_of(a) for a in argument)
-    if isinstance(argument, list):
-        return [_shape_of(a) for a in argument]
-    if isinstance(argument, torch.Tensor):
-        return argument.size()
-    return argument
+        return cls(_describe(tuple(args)), {name: _describe(v) for name, v in kwargs.items()})

@@ -1,57 +1,55 @@
-"""Kernel metrics the wave-scaling strategies read, with the two CUPTI spellings
-the reference's recordings use (analyzer/habitat/analysis/metrics.py:29-88)."""
+"""Kernel metrics the wave-scaling strategies read.  Each has the name CUPTI
+uses from compute capability 7.0 on and the name and unit of the older
+spelling, as in the reference's recordings
+(analyzer/habitat/analysis/metrics.py:29-88)."""
 from enum import Enum
 
 
+def _names_since_volta(device):
+    return device.compute_capability[0] >= 7
+
+
 class _MetricInfo:
-    def __init__(self, cupti_name, legacy_cupti_name, legacy_to_canonical_fn):
-        self._cupti_name = cupti_name
-        self._legacy_cupti_name = legacy_cupti_name
-        self._legacy_to_canonical_fn = legacy_to_canonical_fn
+    __slots__ = ("cupti_name", "legacy_cupti_name", "_legacy_scale")
 
-    @property
-    def cupti_name(self):
-        return self._cupti_name
-
-    @property
-    def legacy_cupti_name(self):
-        return self._legacy_cupti_name
+    def __init__(self, cupti_name, legacy_cupti_name, legacy_scale=None):
+        self.cupti_name = cupti_name
+        self.legacy_cupti_name = legacy_cupti_name
+        self._legacy_scale = legacy_scale    # canonical value = legacy value x this
 
     def to_canonical_value(self, value, device):
-        # Values recorded on compute capability >= 7 are already canonical.
-        if device.compute_capability[0] >= 7:
+        if _names_since_volta(device) or self._legacy_scale is None:
             return value
-        return self._legacy_to_canonical_fn(value)
+        return value * self._legacy_scale
 
 
-def _same(value):
-    return value
+_PCT = ".pct_of_peak_sustained_elapsed"
 
-
-class Metric(Enum):
-    DRAMUtilization = _MetricInfo(
-        "dram__throughput.avg.pct_of_peak_sustained_elapsed", "dram_utilization",
-        lambda value: value * 10)
-    DRAMReadBytes = _MetricInfo("dram__bytes_read.sum", "dram_read_bytes", _same)
-    DRAMWriteBytes = _MetricInfo("dram__bytes_write.sum", "dram_write_bytes", _same)
-    SinglePrecisionFLOPEfficiency = _MetricInfo(
-        "smsp__sass_thread_inst_executed_ops_fadd_fmul_ffma_pred_on.avg."
-        "pct_of_peak_sustained_elapsed", "flop_sp_efficiency", _same)
-    SinglePrecisionAddOps = _MetricInfo(
-        "smsp__sass_thread_inst_executed_op_fadd_pred_on.sum", "flop_count_sp_add", _same)
+Metric = Enum("Metric", {
+    # the old DRAM utilisation is a level 0..10, the new one a percentage
+    "DRAMUtilization": _MetricInfo("dram__throughput.avg" + _PCT, "dram_utilization", 10),
+    "DRAMReadBytes": _MetricInfo("dram__bytes_read.sum", "dram_read_bytes"),
+    "DRAMWriteBytes": _MetricInfo("dram__bytes_write.sum", "dram_write_bytes"),
+    "SinglePrecisionFLOPEfficiency": _MetricInfo(
+        "smsp__sass_thread_inst_executed_ops_fadd_fmul_ffma_pred_on.avg" + _PCT,
+        "flop_sp_efficiency"),
+    "SinglePrecisionAddOps": _MetricInfo(
+        "smsp__sass_thread_inst_executed_op_fadd_pred_on.sum", "flop_count_sp_add"),
+}, module=__name__)
 
 
 def _get_metric_name(metric, device):
-    if isinstance(metric, Metric):
-        info = metric.value
-        return info.cupti_name if device.compute_capability[0] >= 7 else info.legacy_cupti_name
-    return metric
+    if not isinstance(metric, Metric):
+        return metric                        # already a raw name
+    info = metric.value
+    return info.cupti_name if _names_since_volta(device) else info.legacy_cupti_name
 
 
 def resolve_metrics(metrics, device):
-    """Metric enum values -> raw metric names for `device`; raw names pass through."""
+    """Raw metric names for `device` from Metric members (raw names pass
+    through); one metric or a list or tuple of them; None gives []."""
     if metrics is None:
         return []
-    if isinstance(metrics, (list, tuple)):
-        return [_get_metric_name(m, device) for m in metrics]
-    return [_get_metric_name(metrics, device)]
+    if not isinstance(metrics, (list, tuple)):
+        metrics = (metrics,)
+    return [_get_metric_name(metric, device) for metric in metrics]

@@ -1,0 +1,2 @@
+"""Per-operation MLP predictors: model classes and RuntimePredictor (mlp), the
+device-feature table (devices)."""

@@ -1,6 +1,7 @@
 """Run times of one pass (forward or backward) of an operation: measured,
-predicted from kernels, or predicted outright
-(analyzer/habitat/analysis/run_time.py:5-88)."""
+predicted from kernels, or predicted outright.  Same four classes and read-only
+attributes as the reference (analyzer/habitat/analysis/run_time.py:5-88):
+`run_time_ms`, `kernels`, `device` and the kernel-time sum `ktime_ns`."""
 
 
 def ns_to_ms(ns):
@@ -11,79 +12,60 @@ def ms_to_ns(ms):
     return ms * 1e6
 
 
+def _stored(slot):
+    return property(lambda self: getattr(self, slot))
+
+
+def _missing(self):
+    raise NotImplementedError
+
+
 class RunTime:
-    @property
-    def run_time_ms(self):
-        raise NotImplementedError
+    __slots__ = ()
 
-    @property
-    def ktime_ns(self):
-        return sum(k.run_time_ns for k in self.kernels)
-
-    @property
-    def kernels(self):
-        return []
-
-    @property
-    def device(self):
-        raise NotImplementedError
+    run_time_ms = property(_missing)
+    device = property(_missing)
+    kernels = property(lambda self: [])
+    ktime_ns = property(lambda self: sum(kernel.run_time_ns for kernel in self.kernels))
 
 
 class RunTimeMeasurement(RunTime):
+    __slots__ = ("_run_time_ms", "_kernels", "_device")
+
     def __init__(self, run_time_ms, kernels, device):
-        self._run_time_ms = run_time_ms
-        self._kernels = kernels
-        self._device = device
+        self._run_time_ms, self._kernels, self._device = run_time_ms, kernels, device
 
-    @property
-    def run_time_ms(self):
-        return self._run_time_ms
-
-    @property
-    def kernels(self):
-        return self._kernels
-
-    @property
-    def device(self):
-        return self._device
+    run_time_ms = _stored("_run_time_ms")
+    kernels = _stored("_kernels")
+    device = _stored("_device")
 
 
 class RunTimePrediction(RunTime):
-    """overhead + sum of predicted kernel times (run_time.py:42-66)."""
+    """Overhead plus the predicted kernels' times (run_time.py:42-66); the sum
+    is formed on first use and kept."""
+    __slots__ = ("_total_ms", "_overhead_ns", "_predicted_kernels", "_device")
 
     def __init__(self, overhead_ns, predicted_kernels, device):
-        self._run_time_ms = None
+        self._total_ms = None
         self._overhead_ns = overhead_ns
-        self._predicted_kernels = predicted_kernels
-        self._device = device
+        self._predicted_kernels, self._device = predicted_kernels, device
+
+    kernels = _stored("_predicted_kernels")
+    device = _stored("_device")
 
     @property
     def run_time_ms(self):
-        if self._run_time_ms is None:
-            total_ns = self._overhead_ns + sum(k.run_time_ns for k in self.kernels)
-            self._run_time_ms = ns_to_ms(total_ns)
-        return self._run_time_ms
-
-    @property
-    def kernels(self):
-        return self._predicted_kernels
-
-    @property
-    def device(self):
-        return self._device
+        if self._total_ms is None:
+            self._total_ms = ns_to_ms(self._overhead_ns + self.ktime_ns)
+        return self._total_ms
 
 
 class RunTimePurePrediction(RunTime):
     """A predicted time with no kernel breakdown (MLP-predicted operations)."""
+    __slots__ = ("_run_time_ms", "_device")
 
     def __init__(self, run_time_ms, device):
-        self._run_time_ms = run_time_ms
-        self._device = device
+        self._run_time_ms, self._device = run_time_ms, device
 
-    @property
-    def run_time_ms(self):
-        return self._run_time_ms
-
-    @property
-    def device(self):
-        return self._device
+    run_time_ms = _stored("_run_time_ms")
+    device = _stored("_device")
