@@ -138,9 +138,14 @@ class _Device:
         from habitat_amd.data import path_to_data
         with open(path_to_data("devices.yml")) as f:
             table = yaml.safe_load(f)
-        self._devices = {
-            name: DeviceProperties(name=name, **props) for name, props in table.items()
-        }
+        # {columns: [...], devices: {name: row}}, a row being the values in column
+        # order or a mapping; or the reference's layout, {name: mapping}
+        columns = table.get("columns", _FIELDS) if "devices" in table else _FIELDS
+        rows = table["devices"] if "devices" in table else table
+        self._devices = {}
+        for name, row in rows.items():
+            props = row if isinstance(row, dict) else dict(zip(columns, row))
+            self._devices[name] = DeviceProperties(name=name, **props)
 
     def names(self):
         if self._devices is None:

@@ -290,3 +290,25 @@ def test_nothing_in_the_product_imports_the_oracle():
                 if "oracle" in text.replace("oracle's", ""):
                     offenders.append(os.path.join(base, f))
     assert offenders == []
+
+
+def test_device_table_is_read_in_both_layouts(tmp_path, monkeypatch):
+    """The shipped table is columnar; a table in the reference's layout (device
+    names at the top level, one mapping each: analyzer/habitat/data/devices.yml)
+    and rows written as mappings are read the same way."""
+    import yaml
+    import habitat_amd.data
+    from habitat_amd.device import _Device, _FIELDS
+    v100 = {f: getattr(Device.V100, f) for f in ("num_sms", "mem_bandwidth_gb")}
+    as_mapping = dict(Device.V100.as_dict())
+    assert list(as_mapping) == list(_FIELDS)
+    for layout in ({"V100": as_mapping},
+                   {"columns": list(_FIELDS), "devices": {"V100": as_mapping}},
+                   {"columns": list(_FIELDS), "devices": {"V100": list(as_mapping.values())}}):
+        path = tmp_path / "devices.yml"
+        path.write_text(yaml.safe_dump(layout))
+        monkeypatch.setattr(habitat_amd.data, "path_to_data", lambda name: str(path))
+        table = _Device()
+        assert table.names() == ["V100"]
+        assert {f: getattr(table.V100, f) for f in v100} == v100
+        assert table.V100.as_dict() == as_mapping
