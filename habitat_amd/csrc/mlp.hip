@@ -264,6 +264,7 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
 constexpr int kSplit = 8;            // K-partials per hidden layer, up to kRows rows
 constexpr int kLayerMaxRows = 4096;  // largest batch that takes this path
 constexpr int kFewTiles = 8;         // m-tiles up to which the whole-K shape prefetches (DEPTH)
+constexpr int kManyTiles = 32;       // m-tiles from which its workgroups take four n-tiles (NT)
 constexpr size_t kScratchFloats = (size_t)kLayerMaxRows * kWidth;  // each of two buffers
 static_assert((size_t)kSplit * kRows * kWidth <= kScratchFloats, "the K-partials fit the scratch");
 
@@ -288,14 +289,14 @@ struct LayerArgs {
 // G k-groups of a wave: the weight fragments of the n-tile and what the
 // matching activation fragments are made from (the activations themselves, or
 // S_IN K-partials and the bias that goes with them).
-template <int G, int S_IN>
+template <int G, int S_IN, int NT>
 struct LayerFrag {
-  f32x4 w[G];
+  f32x4 w[G][NT];
   f32x4 x[G][S_IN > 0 ? S_IN : 1];
   f32x4 bias[S_IN > 0 ? G : 1];
 };
 
-// One layer for one m-tile (blockIdx.z), one n-tile (blockIdx.x) and one
+// One layer for one m-tile (blockIdx.z), NT n-tiles (blockIdx.x) and one
 // K-partial (blockIdx.y of a.splits).  The WAVES waves split the partial's
 // k-groups (at most G each); fc1 has fewer, so there each group is checked
 // against the wave's count (wave-uniform).
@@ -308,18 +309,22 @@ struct LayerFrag {
 //     padded m-tile holds them) instead of being masked; masking saves most of
 //     the traffic of a handful of rows, not masking keeps the loads of a full
 //     tile free of branches.
+//   NT: n-tiles per workgroup (blockIdx.x counts groups of NT); an activation
+//     fragment then serves NT MFMAs.  Measured for the whole-K shape at 512 /
+//     1024 / 4096 rows: 1: 131 214 753 us; 2: 126 201 704; 4: 188 192 685.
 //   DEPTH: k-groups whose loads are kept in flight ahead of the MFMAs; 0 leaves
 //     the placement to the compiler.  Measured for the whole-K shape (us per
 //     forward at 64 / 256 / 512 / 4096 rows): 0: 80 88 132 766; 2: 70 77 137
 //     841; 4: 76 83 154 1014; 8: 90 97 188 1338; all 16: 95 102 178 1199.  More
 //     loads in flight only crowd the path from L2 once every compute unit has
 //     several workgroups; with a few m-tiles two groups ahead is best.
-template <bool FIRST, int S_IN, bool FINAL, int WAVES, bool PADDED_ROWS, int DEPTH>
+template <bool FIRST, int S_IN, bool FINAL, int WAVES, bool PADDED_ROWS, int DEPTH, int NT = 1>
 __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a) {
+  static_assert(8 % NT == 0, "a workgroup's n-tiles lie in one wave stream of the packed weights");
   static_assert(S_IN == 0 || !FINAL, "K-partials go in and come out together");
   static_assert(WAVES == 4 || WAVES == 8, "the reduction below is written for these");
   constexpr int G = FIRST ? kMaxInPadded / 8 / WAVES : kWidth / 8 / WAVES / (FINAL ? 1 : kSplit);
-  __shared__ float red[WAVES][16][64];
+  __shared__ float red[WAVES][NT][16][64];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -338,17 +343,18 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
   count = count < 0 ? 0 : (count > per_wave ? per_wave : count);
 
   // n-tile of the layer -> (stream of the fused kernel's wave, slot in its group)
-  const int tile = blockIdx.x;
+  const int tile = blockIdx.x * NT;  // the first of the workgroup's NT
   const f32x4* w_lane = reinterpret_cast<const f32x4*>(a.w_stream) +
                         ((size_t)(tile >> 3) * a.groups_total + a.g0) * (8 * 64) +
                         (tile & 7) * 64 + lane;
 
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-  LayerFrag<G, S_IN> f;
+  LayerFrag<G, S_IN, NT> f;
   auto load_group = [&](int j) {
     if (!FIRST || j < count) {
       const int gl = first + j;  // layer-local group
-      f.w[j] = w_lane[(size_t)gl * (8 * 64)];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) f.w[j][t] = w_lane[(size_t)gl * (8 * 64) + t * 64];
       const int k = 8 * gl + 4 * h;
       if (FIRST) {
         f32x4 v = zero;
@@ -375,9 +381,11 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
     }
   };
 
-  f32x16 acc;
+  f32x16 acc[NT];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
   auto mfma_group = [&](int j) {
     if (!FIRST || j < count) {
       f32x4 v = f.x[j][0];
@@ -391,7 +399,9 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(f.w[j][e], v[e], acc, 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.w[j][t][e], v[e], acc[t], 0, 0, 0);
     }
   };
 
@@ -416,28 +426,33 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
   }
 
 #pragma unroll
-  for (int r = 0; r < 16; ++r) red[wave][r][lane] = acc[r];
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[wave][t][r][lane] = acc[t][r];
   __syncthreads();
   // thread (wave, lane) adds the waves' registers R*wave .. R*wave+R-1, in wave
   // order: accumulator register 4g + e of lane (m, h) is output n = 8g + 4h + e
   // of row m
   constexpr int R = 16 / WAVES;
   const int r0 = R * wave;
-  const int n0 = tile * 32 + 8 * (r0 >> 2) + 4 * h + (r0 & 3);
-  float o[R];
 #pragma unroll
-  for (int e = 0; e < R; ++e) {
-    float sum = red[0][r0 + e][lane];
+  for (int t = 0; t < NT; ++t) {
+    const int n0 = (tile + t) * 32 + 8 * (r0 >> 2) + 4 * h + (r0 & 3);
+    float o[R];
 #pragma unroll
-    for (int w = 1; w < WAVES; ++w) sum += red[w][r0 + e][lane];
-    if (FINAL) sum = fmaxf(sum + a.bias_out[n0 + e], 0.f);
-    o[e] = sum;
-  }
-  float* dst = a.p_out + ((size_t)split * a.m_pad + (size_t)blockIdx.z * kRows + m) * kWidth + n0;
-  if constexpr (R == 4) {
-    *reinterpret_cast<f32x4*>(dst) = f32x4{o[0], o[1], o[2], o[3]};
-  } else {
-    *reinterpret_cast<f32x2*>(dst) = f32x2{o[0], o[1]};
+    for (int e = 0; e < R; ++e) {
+      float sum = red[0][t][r0 + e][lane];
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) sum += red[w][t][r0 + e][lane];
+      if (FINAL) sum = fmaxf(sum + a.bias_out[n0 + e], 0.f);
+      o[e] = sum;
+    }
+    float* dst = a.p_out + ((size_t)split * a.m_pad + (size_t)blockIdx.z * kRows + m) * kWidth + n0;
+    if constexpr (R == 4) {
+      *reinterpret_cast<f32x4*>(dst) = f32x4{o[0], o[1], o[2], o[3]};
+    } else {
+      *reinterpret_cast<f32x2*>(dst) = f32x2{o[0], o[1]};
+    }
   }
 }
 
@@ -568,6 +583,9 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
     else if (!split_k && m_tiles <= kFewTiles)
       hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 2>), grid, dim3(512), 0,
                          stream, l);
+    else if (!split_k && m_tiles >= kManyTiles)
+      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 0, 4>),
+                         dim3(kWidth / 128, 1, (unsigned)m_tiles), dim3(512), 0, stream, l);
     else if (!split_k)
       hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 0>), grid, dim3(512), 0,
                          stream, l);
