@@ -47,13 +47,6 @@ enum {
 };
 
 /*
- * Device description.  Replaces habitat::cuda::DeviceProperties
- * (cpp/src/cuda/kernel.h:14-62; Python constructor
- * cpp/src/frontend/model_bindings.cpp:17-55) minus the name, which stays on
- * the host side.  The three double fields hold integer values, as the
- * reference's fields are integers (kernel.h:59-61).
- */
-/*
  * compute_major of a device described by AMD's compute-unit model instead of
  * the reference's NVIDIA one: 100 + the major HIP reports for the gfx9 family
  * (compute_minor = HIP's minor: 0 gfx90a, 4 gfx942, 5 gfx950).  No counterpart
@@ -71,6 +64,13 @@ enum {
  */
 #define HBT_COMPUTE_MAJOR_CDNA 109
 
+/*
+ * Device description.  Replaces habitat::cuda::DeviceProperties
+ * (cpp/src/cuda/kernel.h:14-62; Python constructor
+ * cpp/src/frontend/model_bindings.cpp:17-55) minus the name, which stays on
+ * the host side.  The three double fields hold integer values, as the
+ * reference's fields are integers (kernel.h:59-61).
+ */
 typedef struct hbt_device_spec {
   int32_t compute_major, compute_minor;
   int32_t max_threads_per_block, max_threads_per_sm;
