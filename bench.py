@@ -12,6 +12,8 @@ inputs resident in HBM.  Prints ONE JSON line:
                 launch stream)
   cpu_baseline  the CPU oracle (C restatement of the reference's per-kernel
                 Python, one thread) on the same records, same machine
+  multi_destination  the same records scaled to the seven other NVIDIA devices of the
+                device table in one launch (records read once)
   large         the same kernel at 64 M records (beyond the 256 MB last-level cache);
                 large_16M: at 16 M records
   mlp           the fused MFMA MLP (configs[2], conv2d, 1 M rows): rows/s, its
@@ -76,15 +78,18 @@ class WaveScaleCall:
     measures the library and the GPU rather than Python argument handling."""
 
     def __init__(self, records, origin, dest, out):
+        """`dest`: one device, or a list of them (outputs [n_dest][n])."""
         import torch
         from habitat_amd import _lib
         self.lib = _lib.lib()
-        self.keep = (records, out, origin, dest)
+        dests = dest if isinstance(dest, (list, tuple)) else [dest]
+        specs = (_lib.DeviceSpec * len(dests))(*[d.spec for d in dests])
+        self.keep = (records, out, origin, dests, specs)
         p = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
         c = records.columns
         self.stream = torch.cuda.current_stream()
         self.args = (
-            ctypes.byref(origin.spec), ctypes.byref(dest.spec), 1, records.n,
+            ctypes.byref(origin.spec), specs, len(dests), records.n,
             p(c["num_blocks"]), p(c["block_size"]), p(c["dynamic_smem"]), p(c["static_smem"]),
             p(c["regs_per_thread"]), p(records.dest_regs), p(c["run_time_ns"]),
             p(c["flop_sp_efficiency"]), p(c["dram_read_bytes"]), p(c["dram_write_bytes"]),
@@ -426,6 +431,25 @@ def main():
                 "roofline": {"bound": "hbm", "achieved": b_ach, "peak": HBM_PEAK_GBS,
                              "unit": "GB/s", "frac": b_ach / HBM_PEAK_GBS,
                              "launch_us": b_launch * 1e3}}
+
+    # ---------------- the same records for every other NVIDIA device of the table ------------
+    def multi_dest_section():
+        dests = [getattr(Device, name) for name in Device.names()
+                 if name != origin.name and not name.startswith("MI355X")]
+        m_out = WaveScaleOutput(records.n, len(dests), records.device, waves=False, status=True)
+        m_call = WaveScaleCall(records, origin, dests, m_out)
+        m_wall, m_launch = time_steps(m_call, max(args.steps // 4, 5), max(args.warmup // 4, 2))
+        per_record = 52 + 17 * len(dests)     # the record is read once per launch
+        gbs = per_record * records.n / (m_launch * 1e-3) / 1e9
+        return {"destinations": [d.name for d in dests], "launch_us": m_launch * 1e3,
+                "us_per_destination": m_launch * 1e3 / len(dests),
+                "value": records.n * len(dests) / (m_wall * 1e-3),
+                "unit": "(record, destination) pairs/s",
+                "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": gbs / HBM_PEAK_GBS, "bytes_per_record": per_record}}
+
+    if not args.no_large:
+        attempt("multi_destination", multi_dest_section)
 
     del call, records, out
     if not args.no_large and args.large_records > args.records:
