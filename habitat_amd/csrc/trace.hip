@@ -105,7 +105,9 @@ __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a)
   RecordMid m = origin_part<MODEL>(a.origin, r);
   if (__builtin_expect(m.redo_gflops, 0))
     m.num_gflops = origin_gflops_exact(a.origin.peak_gflops, r.eff, r.t);
-  const RecordOut o = dest_part<MODEL, false>(p, r, m, 0.0);
+  RecordOut o = dest_part<MODEL, false>(p, r, m, 0.0);
+  if (__builtin_expect(o.in_order, 0))
+    o.t = scaled_time_in_order(r.t, o.gamma, p.log2_bw, p.log2_clk, p.log2_clk_sm);
 
   const bool ok = in_range && o.status == HBT_ST_OK;
   double v = ok ? o.t : 0.0;

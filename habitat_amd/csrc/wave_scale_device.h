@@ -212,8 +212,22 @@ __device__ __noinline__ double origin_gflops_exact(double peak_gflops, double ef
   return gflops_per_second * t / 1e9;
 }
 
+// t * bw^gamma * clk^(1-gamma) * sm^(1-gamma) multiplied out from left to right
+// as the reference does (roofline.py:58-63), for run times so large that a
+// partial product overflows where the whole product does not: the reference
+// then returns inf, and so must this.
+__device__ __noinline__ double scaled_time_in_order(double t, double gamma, double log2_bw,
+                                                    double log2_clk, double log2_clk_sm) {
+  const double gamma_compl = 1.0 - gamma;
+  double v = t * exp2_poly(gamma * log2_bw);
+  v = v * exp2_poly(gamma_compl * log2_clk);
+  return v * exp2_poly(gamma_compl * (log2_clk_sm - log2_clk));
+}
+
 struct RecordOut {
   double t;
+  double gamma;
+  bool in_order;  // t must be replaced by scaled_time_in_order (see there)
   int32_t occ_d, wave_d;
   uint8_t status;
 };
@@ -289,6 +303,15 @@ __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn
                           gamma_compl * (small ? log2_small : p.log2_clk_sm);
   const double t = r.t * exp2_poly(exponent);
   o.t = (status == HBT_ST_OK) ? t : __builtin_nan("");
+  // One combined power is the product of the reference's three to rounding,
+  // unless a partial product overflows on the way where the whole does not:
+  // only possible for run times beyond 2^500 ns (the factors are ratios of
+  // device constants).  Those are left to the caller (scaled_time_in_order), so
+  // that this function stays free of branches.  (No such case at the other
+  // end: with a time small enough to underflow the FLOP count falls below
+  // 1e-9, gamma is 1 and one factor is left.)
+  o.gamma = gamma;
+  o.in_order = status == HBT_ST_OK && !small && fabs(r.t) > 0x1p500;
   return o;
 }
 

@@ -132,6 +132,23 @@ def test_scaling_closed_forms(kat):
     r_hi = _record(kat, big, dram_read_bytes=nbytes * (1 - 1e-9), dram_write_bytes=0.0)
     assert ows.gamma(r_lo, v100, p100) == pytest.approx(0.5, abs=1e-8)
     assert ows.gamma(r_hi, v100, p100) == pytest.approx(0.5, abs=1e-8)
+    # The three factors are multiplied onto the time from left to right
+    # (roofline.py:58-63), so a partial product may leave the range of fp64
+    # where the whole product does not.  No bytes: gamma = 0, factors 1, clock
+    # ratio, SM ratio.  RTX2070 -> V100: 1.7e308 * (1410/1312) overflows before
+    # 36/80 brings it back.  (Nothing of the kind at the other end of the range:
+    # a time small enough to underflow makes the FLOP count fall below 1e-9,
+    # which forces gamma = 1 and leaves one factor.)
+    no_bytes = dict(dram_read_bytes=0.0, dram_write_bytes=0.0)
+    rtx2070 = oracle_device(DEVS["RTX2070"])
+    for t_in, want in ((1.7e308, math.inf), (1e300, 1e300 * (1410 / 1312) * (36 / 80))):
+        r = _record(kat, big, run_time_ns=t_in, **no_bytes)
+        assert ows.gamma(r, rtx2070, v100) == 0.0
+        assert ows.unified(r, rtx2070, v100) == pytest.approx(want, rel=1e-15)
+        c = olib.wave_scale(rtx2070, v100, _cols([r]))
+        assert c["status"][0] == 0 and c["time_ns"][0] == pytest.approx(want, rel=1e-15)
+    tiny = _record(kat, big, run_time_ns=5e-324, **no_bytes)
+    assert ows.gamma(tiny, oracle_device(DEVS["T4"]), oracle_device(DEVS["P4000"])) == 1.0
     # without metrics: small kernel unchanged, else bandwidth ratio
     assert ows.unified(_record(kat, 3), v100, p100, has_metrics=False) == 1000000
     assert ows.unified(_record(kat, big), v100, p100, has_metrics=False) == pytest.approx(

@@ -170,6 +170,49 @@ def test_adversarial_field_values_agree_with_the_oracle_bit_for_bit_in_status():
         np.testing.assert_allclose(t[plain], w[plain], rtol=TIME_RTOL, atol=0)
 
 
+def test_partial_products_overflow_as_in_the_reference():
+    """The reference multiplies t by its three factors from left to right, so
+    1.7e308 ns * 1.07 is already inf when 0.45 follows; the kernel's single
+    combined power must not return the finite product there.  Huge and ordinary
+    times, every device pair, single and multi-destination launches."""
+    rng = np.random.default_rng(8)
+    rec, _ = synthetic.kernel_records(30_000, Device.V100, seed=41, metrics_fraction=0.8)
+    rec["run_time_ns"] = np.where(rng.random(30_000) < 0.5, rec["run_time_ns"],
+                                  rng.choice([1.7e308, 1e308, 4e307, 1e305, 1e200, 3.3e150,
+                                              1e151, np.inf], 30_000))
+    rec["dram_read_bytes"] = np.where(rng.random(30_000) < 0.3, 0.0, rec["dram_read_bytes"])
+    rec["dram_write_bytes"] = np.where(rng.random(30_000) < 0.5, 0.0, rec["dram_write_bytes"])
+    kr = KernelRecords.from_numpy(rec)
+    names = ["RTX2070", "V100", "T4", "P4000", "P100", "MI355X"]
+    devices = [getattr(Device, n) for n in names]
+    n_inf_where_product_is_finite = 0
+    for origin in devices:
+        multi = wave_scale(kr, origin, devices)
+        for d, dest in enumerate(devices):
+            want = olib.wave_scale(odev(origin), odev(dest), rec)
+            single = wave_scale(kr, origin, [dest])
+            for out, row in ((multi, d), (single, 0)):
+                st = out.status[row].cpu().numpy()
+                assert np.array_equal(st, want["status"])
+                t, w = out.time_ns[row].cpu().numpy(), want["time_ns"]
+                ok = st == 0
+                assert np.array_equal(np.isinf(t[ok]), np.isinf(w[ok])), (origin.name, dest.name)
+                fin = ok & np.isfinite(w)
+                np.testing.assert_allclose(t[fin], w[fin], rtol=TIME_RTOL, atol=0)
+            n_inf_where_product_is_finite += int(np.sum(
+                (want["status"] == 0) & np.isinf(want["time_ns"]) & np.isfinite(rec["run_time_ns"])))
+    assert n_inf_where_product_is_finite > 1000
+    # the hand-checked case: no bytes, gamma = 0, RTX2070 -> V100
+    one = {k: v[:1].copy() for k, v in rec.items()}
+    one.update(num_blocks=np.array([1 << 16], np.int32), run_time_ns=np.array([1.7e308]),
+               dram_read_bytes=np.array([0.0]), dram_write_bytes=np.array([0.0]),
+               has_metrics=np.array([1], np.uint8), block_size=np.array([256], np.int32),
+               regs_per_thread=np.array([32], np.int32), static_smem=np.array([0], np.int32),
+               dynamic_smem=np.array([0], np.int32), flop_sp_efficiency=np.array([50.0]))
+    out = wave_scale(KernelRecords.from_numpy(one), Device.RTX2070, [Device.V100])
+    assert out.status[0].item() == 0 and out.time_ns[0].item() == math.inf
+
+
 def test_more_than_2_to_28_records_take_64_bit_offsets():
     """Above 2^28 records byte offsets no longer fit 32 bits and the kernel's
     64-bit-offset instantiation runs.  Records are generated on the GPU (19 GB of
