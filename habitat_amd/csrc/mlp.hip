@@ -45,6 +45,11 @@ using f32x2 = float __attribute__((ext_vector_type(2)));
 using f32x4 = float __attribute__((ext_vector_type(4)));
 using f32x16 = float __attribute__((ext_vector_type(16)));
 
+// ReLU that hands a NaN on, as torch's does (a feature that is NaN or infinite,
+// or a zero sigma, must give a NaN prediction as in the reference); the
+// hardware's max would return the other operand, 0.
+__device__ __forceinline__ float relu(float v) { return v < 0.f ? 0.f : v; }
+
 constexpr int kWidth = 1024;      // hidden width the kernel is built for
 constexpr int kRows = 32;         // rows per workgroup (one MFMA tile of m)
 constexpr int kStride = kWidth + 4;  // LDS row stride in floats
@@ -162,6 +167,8 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
     }
     act[r * kStride + k] = v;
   }
+  // fc1's bias, where the accumulators will pick it up
+  *reinterpret_cast<f32x4*>(bias_lds + 4 * tid) = *reinterpret_cast<const f32x4*>(a.bias + 4 * tid);
   __syncthreads();
 
   const float* act_lane = act + m * kStride + 4 * h;
@@ -181,31 +188,38 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
   f32x16 acc[TPW];
   int g0 = 0;
   for (int layer = 0; layer <= a.hidden; ++layer) {
-    // This layer's bias goes through LDS: every thread fetches four values now
-    // and parks them in LDS after the K loop, so that the write-back below
-    // finds them without waiting for global memory.
+    // The accumulators start at this layer's bias, which the layer before
+    // parked in LDS; every thread fetches four values of the next layer's now
+    // and parks them after the K loop.  (Adding the bias here instead of in the
+    // write-back leaves room there for a ReLU that hands NaNs on, at no more
+    // instructions than add and max.)
+    const int next_layer = layer < a.hidden ? layer + 1 : layer;
     const f32x4 bias_part =
-        *reinterpret_cast<const f32x4*>(a.bias + (size_t)layer * kWidth + 4 * tid);
+        *reinterpret_cast<const f32x4*>(a.bias + (size_t)next_layer * kWidth + 4 * tid);
 #pragma unroll
     for (int t = 0; t < TPW; ++t)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 b =
+            *reinterpret_cast<const f32x4*>(bias_lds + (tile0 + t) * 32 + 8 * g + 4 * h);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[t][4 * g + e] = b[e];
+      }
 
     const int kg = (layer == 0) ? kg_first : kWidth / 8;
     layer_k_loop<TPW>(ring, stream, g0, kg, g_end, act_lane, acc);
     g0 += kg;
 
+    __syncthreads();  // every wave has finished reading this layer's input and bias
     *reinterpret_cast<f32x4*>(bias_lds + 4 * tid) = bias_part;
-    __syncthreads();  // every wave has finished reading this layer's input
 #pragma unroll
     for (int t = 0; t < TPW; ++t)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int n = (tile0 + t) * 32 + 8 * g + 4 * h;
-        const f32x4 b = *reinterpret_cast<const f32x4*>(bias_lds + n);
         f32x4 o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = fmaxf(acc[t][4 * g + e] + b[e], 0.f);
+        for (int e = 0; e < 4; ++e) o[e] = relu(acc[t][4 * g + e]);
         *reinterpret_cast<f32x4*>(act + m * kStride + n) = o;
       }
     __syncthreads();
@@ -395,7 +409,7 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
 #pragma unroll
         for (int s = 0; s < S_IN; ++s) v += f.x[j][s];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = fmaxf(v[e], 0.f);
+        for (int e = 0; e < 4; ++e) v[e] = relu(v[e]);
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e)
@@ -444,7 +458,7 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
       float sum = red[0][t][r0 + e][lane];
 #pragma unroll
       for (int w = 1; w < WAVES; ++w) sum += red[w][t][r0 + e][lane];
-      if (FINAL) sum = fmaxf(sum + a.bias_out[n0 + e], 0.f);
+      if (FINAL) sum = relu(sum + a.bias_out[n0 + e]);
       o[e] = sum;
     }
     float* dst = a.p_out + ((size_t)split * a.m_pad + (size_t)blockIdx.z * kRows + m) * kWidth + n0;
@@ -490,7 +504,7 @@ __global__ __launch_bounds__(256) void mlp_last_kernel(const LastArgs a) {
 #pragma unroll
       for (int s = 0; s < S_IN; ++s) v += part[i][s];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = fmaxf(v[e], 0.f);
+      for (int e = 0; e < 4; ++e) v[e] = relu(v[e]);
     }
     const f32x4 wl = *reinterpret_cast<const f32x4*>(a.w_last + k);
 #pragma unroll

@@ -274,3 +274,36 @@ def test_config2_and_config3_full_size_properties(kind):
     assert torch.equal(y_perm[fused_both], y[perm][fused_both])
     assert torch.allclose(y_perm, y[perm], rtol=1e-5, atol=1e-7)
     assert bool(torch.all(torch.isfinite(y)))
+
+
+@pytest.mark.parametrize("zero_sigma", [False, True])
+def test_nan_and_infinite_features_give_what_torch_gives(zero_sigma):
+    """A feature that is NaN or infinite, or a sigma of zero (a constant column
+    in the training set), makes the reference's torch forward return NaN for
+    that row: ReLU hands a NaN on there, where the hardware's max would return
+    0.  Same rows through the three paths; the other rows stay within the
+    tolerance."""
+    rp = make("conv2d")
+    x, mu, sigma = synthetic.mlp_features("conv2d", 9000, seed=2)
+    rng = np.random.default_rng(1)
+    x = x.copy()
+    special = np.array([np.nan, np.inf, -np.inf, 1e300, -1e300, 3e38, 1e-300, 0.0])
+    for r in rng.choice(9000, 900, replace=False):
+        x[r, rng.integers(0, x.shape[1])] = rng.choice(special)
+    if zero_sigma:
+        sigma = np.where(np.arange(sigma.shape[0]) == 3, 0.0, sigma)
+    rp.set_normalization(mu, sigma)
+    sd = rp.model.state_dict()
+    for rows in (20, 300, 9000):
+        with np.errstate(all="ignore"):
+            want = omlp.forward_fp32(sd, x[:rows], mu, sigma)
+        got = rp.predict_batch(x[:rows]).cpu().numpy()
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(np.isposinf(got), np.isposinf(want))
+        assert np.array_equal(np.isneginf(got), np.isneginf(want))
+        fin = np.isfinite(want)
+        assert zero_sigma or (fin.sum() > 0.9 * rows and (~fin).sum() > 0.04 * rows) or rows == 20
+        # fp32 against fp32 here: two summation orders of the same numbers
+        assert np.all(np.abs(got[fin] - want[fin]) <= 1e-4 * np.maximum(np.abs(want[fin]), 1e-3))
+    if zero_sigma:
+        assert np.all(np.isnan(want))
