@@ -41,6 +41,7 @@ namespace hbt {
 
 namespace {
 
+using u32x4 = unsigned int __attribute__((ext_vector_type(4)));
 using f32x2 = float __attribute__((ext_vector_type(2)));
 using f32x4 = float __attribute__((ext_vector_type(4)));
 using f32x16 = float __attribute__((ext_vector_type(16)));
@@ -80,12 +81,32 @@ struct Ring {
   f32x4 x[4];
 };
 
+// The wave's weight stream as a buffer resource: a load then takes the stream's
+// base from scalar registers, the k-group's offset as a scalar and the lane's
+// 16 bytes as one 32-bit register, with no 64-bit address arithmetic.
+struct WeightStream {
+  __amdgpu_buffer_rsrc_t rsrc;
+  int lane_bytes;  // 16 * lane
+};
+
+__device__ __forceinline__ WeightStream weight_stream(const f32x4* stream, int64_t bytes,
+                                                      int lane) {
+  WeightStream w;
+  w.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<f32x4*>(stream), 0, (int)bytes, 0x00020000);
+  w.lane_bytes = 16 * lane;
+  return w;
+}
+
 template <int TPW, int SLOT>
-__device__ __forceinline__ void ring_load_w(Ring<TPW>& r, const f32x4* __restrict__ stream,
-                                            int group, int lane) {
-  const f32x4* p = stream + (size_t)group * TPW * 64 + lane;
+__device__ __forceinline__ void ring_load_w(Ring<TPW>& r, const WeightStream& stream, int group,
+                                            int lane) {
+  const int group_bytes = group * (TPW * 64 * 16);
 #pragma unroll
-  for (int t = 0; t < TPW; ++t) r.w[SLOT][t] = p[t * 64];
+  for (int t = 0; t < TPW; ++t) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(stream.rsrc, stream.lane_bytes + t * 1024,
+                                                          group_bytes, 0);
+    r.w[SLOT][t] = __builtin_bit_cast(f32x4, v);
+  }
 }
 
 template <int TPW, int SLOT>
@@ -106,7 +127,7 @@ __device__ __forceinline__ void ring_mfma(const Ring<TPW>& r, f32x16 (&acc)[TPW]
 // group `g0` of the wave's stream; `g_end` is the stream's last valid group.
 // On entry ring slots 0..2 hold the weights of groups g0..g0+2.
 template <int TPW>
-__device__ __forceinline__ void layer_k_loop(Ring<TPW>& r, const f32x4* __restrict__ stream,
+__device__ __forceinline__ void layer_k_loop(Ring<TPW>& r, const WeightStream& stream,
                                              int g0, int kg, int g_end, const float* act_lane,
                                              f32x16 (&acc)[TPW]) {
   const int lane = threadIdx.x & 63;
@@ -177,7 +198,11 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
   // This wave's weight stream: fc1's groups, then 128 groups per hidden layer.
   const int kg_first = a.in_padded / 8;
   const int groups = kg_first + a.hidden * (kWidth / 8);
-  const f32x4* stream = reinterpret_cast<const f32x4*>(a.w_stream) + (size_t)wave * groups * TPW * 64;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int64_t stream_bytes = (int64_t)groups * TPW * 64 * 16;
+  const WeightStream stream = weight_stream(
+      reinterpret_cast<const f32x4*>(a.w_stream) + (size_t)wave_u * groups * TPW * 64, stream_bytes,
+      lane);
   const int g_end = groups - 1;
 
   Ring<TPW> ring;
