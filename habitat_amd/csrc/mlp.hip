@@ -389,34 +389,55 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
 
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   LayerFrag<G, S_IN, NT> f;
+  // Hidden layers fetch weights, activations (or K-partials) and bias through
+  // buffer loads: bases in scalar registers, the k-group's offset a scalar, one
+  // 32-bit register of lane offset each, no 64-bit address arithmetic.  A lane
+  // whose row is past the end of the batch gets an offset beyond the buffer
+  // instead of a branch around the load: such a load returns zeros.
+  constexpr bool BUFFER = !FIRST;
+  __amdgpu_buffer_rsrc_t w_rsrc, x_rsrc, b_rsrc;
+  int w_lane_bytes = 0, x_lane_bytes = 0, w_base_bytes = 0;
+  const int split_bytes = a.m_pad * (kWidth * 4);  // one K-partial, or the activations
+  if (BUFFER) {
+    w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.w_stream), 0,
+                                               4 * a.groups_total * (8 * 64 * 16), 0x00020000);
+    x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.p_in), 0,
+                                               (S_IN > 0 ? S_IN : 1) * split_bytes, 0x00020000);
+    b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.bias_in), 0, kWidth * 4,
+                                               0x00020000);
+    w_lane_bytes = ((tile & 7) * 64 + lane) * 16;
+    w_base_bytes = ((tile >> 3) * a.groups_total + a.g0) * (8 * 64 * 16);
+    x_lane_bytes = row_ok ? (int)row * (kWidth * 4) + 16 * h : 0x7fffff00;
+  }
   auto load_group = [&](int j) {
     if (!FIRST || j < count) {
       const int gl = first + j;  // layer-local group
+      if (BUFFER) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          f.w[j][t] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+              w_rsrc, w_lane_bytes + t * 1024, w_base_bytes + gl * (8 * 64 * 16), 0));
+#pragma unroll
+        for (int s = 0; s < (S_IN > 0 ? S_IN : 1); ++s)
+          f.x[j][s] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+              x_rsrc, x_lane_bytes, s * split_bytes + gl * 32, 0));
+        if (S_IN > 0)
+          f.bias[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+              b_rsrc, 16 * h, gl * 32, 0));
+        return;
+      }
+      // fc1: a few groups, the raw fp64 features standardised on the spot
 #pragma unroll
       for (int t = 0; t < NT; ++t) f.w[j][t] = w_lane[(size_t)gl * (8 * 64) + t * 64];
       const int k = 8 * gl + 4 * h;
-      if (FIRST) {
-        f32x4 v = zero;
-        if (row_ok) {
+      f32x4 v = zero;
+      if (row_ok) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (k + e < a.in_features)
-              v[e] = (float)((a.raw[row * a.in_features + k + e] - a.mu[k + e]) / a.sigma[k + e]);
-        }
-        f.x[j][0] = v;
-      } else if (S_IN == 0) {
-        f.x[j][0] = zero;
-        if (row_ok) f.x[j][0] = *reinterpret_cast<const f32x4*>(a.p_in + (size_t)row * kWidth + k);
-      } else {
-#pragma unroll
-        for (int s = 0; s < S_IN; ++s) f.x[j][s] = zero;
-        if (row_ok) {
-#pragma unroll
-          for (int s = 0; s < S_IN; ++s)
-            f.x[j][s] = *reinterpret_cast<const f32x4*>(a.p_in + ((size_t)s * a.m_pad + row) * kWidth + k);
-        }
-        f.bias[j] = *reinterpret_cast<const f32x4*>(a.bias_in + k);
+        for (int e = 0; e < 4; ++e)
+          if (k + e < a.in_features)
+            v[e] = (float)((a.raw[row * a.in_features + k + e] - a.mu[k + e]) / a.sigma[k + e]);
       }
+      f.x[j][0] = v;
     }
   };
 
