@@ -16,7 +16,6 @@ import numpy as np
 import torch
 
 from habitat_amd.analysis import SPECIAL_OPERATIONS
-from habitat_amd.analysis.kernels import PredictedKernel
 from habitat_amd.analysis.metrics import Metric
 from habitat_amd.analysis.mlp.devices import get_device_features
 from habitat_amd.analysis.mlp.mlp import RuntimePredictor
@@ -232,49 +231,52 @@ class Predictor:
         by_origin = {}
         for idx, rt in enumerate(run_times):
             by_origin.setdefault(rt.device.name, (rt.device, []))[1].append(idx)
-        times = [None] * len(run_times)
+        out = [None] * len(run_times)
         for origin, idxs in by_origin.values():
-            kernels = [k for idx in idxs for k in run_times[idx].kernels]
-            if kernels:
-                rec = self._records_of([run_times[idx] for idx in idxs], kernels, dest_device,
-                                       mode)
+            passes = [run_times[idx] for idx in idxs]
+            rec, measured_ns, overheads_ns = self._records_of(passes, dest_device, mode)
+            t = []
+            if measured_ns:
                 res = wave_scale(rec, occupancy_device(origin, mode),
                                  [occupancy_device(dest_device, mode)], waves=False)
                 t = res.time_ns[0].cpu().tolist()
                 st = res.status[0].cpu().numpy()
-                bad = np.flatnonzero(st)
-                if bad.size:
-                    raise_for_status(int(st[bad[0]]))
-            pos = 0
-            for idx in idxs:
-                ks = run_times[idx].kernels
+                if st.any():
+                    raise_for_status(int(st[np.flatnonzero(st)[0]]))
                 # an unchanged time keeps the measured value's own type (an int)
-                times[idx] = [k.run_time_ns if v == k.run_time_ns else v
-                              for k, v in zip(ks, t[pos:pos + len(ks)])]
+                t = [m if v == m else v for m, v in zip(measured_ns, t)]
+            pos = 0
+            for idx, rt, overhead_ns in zip(idxs, passes, overheads_ns):
+                ks = rt.kernels
+                out[idx] = RunTimePrediction.from_times(overhead_ns, ks, t[pos:pos + len(ks)],
+                                                        dest_device)
                 pos += len(ks)
-        for rt, vals in zip(run_times, times):
-            preds = [PredictedKernel(k, v) for k, v in zip(rt.kernels, vals)]
-            out.append(self._assemble(rt, preds, dest_device))
         return out
 
-    def _records_of(self, passes, kernels, dest_device, mode):
-        """The kernel records of `passes` as columns on the GPU.  The last few
-        sets are kept (keyed by the identity of the measured passes, which this
-        package treats as immutable once measured), so that predicting one trace
-        for one destination after another converts and uploads its kernels once.
-        The register column depends on the destination's architecture only."""
+    def _records_of(self, passes, dest_device, mode):
+        """(kernel records of `passes` as columns on the GPU, the kernels'
+        measured times, each pass's overhead).  The last few sets are kept
+        (keyed by the identity of the measured passes, which this package treats
+        as immutable once measured), so that predicting one trace for one
+        destination after another converts and uploads its kernels once.  The
+        register column depends on the destination's architecture only."""
         lut = not isinstance(self._kernel_metadata, NullMetadataManager)
         key = (tuple(id(p) for p in passes), mode, dest_device.compute_capability if lut else None,
                torch.cuda.current_device())
         hit = self._record_cache.get(key)
         if hit is not None:
             self._record_cache.move_to_end(key)
-            return hit[0]
-        rec = records_from_kernels(kernels, dest_device, self._kernel_metadata, mode)
-        self._record_cache[key] = (rec, list(passes))   # the passes stay alive with their ids
+            return hit[:3]
+        kernels = [k for p in passes for k in p.kernels]
+        rec = (records_from_kernels(kernels, dest_device, self._kernel_metadata, mode)
+               if kernels else None)
+        measured_ns = [k.run_time_ns for k in kernels]
+        overheads_ns = [self._overhead_ns(p) for p in passes]
+        # the passes stay alive with their ids
+        self._record_cache[key] = (rec, measured_ns, overheads_ns, list(passes))
         while len(self._record_cache) > self._RECORD_CACHE_SETS:
             self._record_cache.popitem(last=False)
-        return rec
+        return rec, measured_ns, overheads_ns
 
     def clear_record_cache(self):
         """Forget the cached kernel-record columns (after changing a measured
@@ -282,10 +284,15 @@ class Predictor:
         self._record_cache.clear()
 
     @staticmethod
-    def _assemble(run_time, predicted_kernels, dest_device):
-        run_time_ns = ms_to_ns(run_time.run_time_ms)
-        overhead_ns = run_time_ns - sum(k.run_time_ns for k in run_time.kernels)
-        return RunTimePrediction(overhead_ns=0 if overhead_ns < 0 else overhead_ns,
+    def _overhead_ns(run_time):
+        """What a measured pass took beyond its kernels, never negative
+        (predictor.py:126-130)."""
+        overhead_ns = ms_to_ns(run_time.run_time_ms) - sum(k.run_time_ns for k in run_time.kernels)
+        return 0 if overhead_ns < 0 else overhead_ns
+
+    @classmethod
+    def _assemble(cls, run_time, predicted_kernels, dest_device):
+        return RunTimePrediction(overhead_ns=cls._overhead_ns(run_time),
                                  predicted_kernels=predicted_kernels, device=dest_device)
 
     def _special_scale_many(self, kind, operations, dest_device):

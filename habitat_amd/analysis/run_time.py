@@ -42,16 +42,39 @@ class RunTimeMeasurement(RunTime):
 
 class RunTimePrediction(RunTime):
     """Overhead plus the predicted kernels' times (run_time.py:42-66); the sum
-    is formed on first use and kept."""
-    __slots__ = ("_total_ms", "_overhead_ns", "_predicted_kernels", "_device")
+    is formed on first use and kept.  `from_times` makes one from the measured
+    kernels and their predicted times, and wraps each pair in a PredictedKernel
+    only when `kernels` is read."""
+    __slots__ = ("_total_ms", "_overhead_ns", "_predicted_kernels", "_device", "_measured",
+                 "_times")
 
     def __init__(self, overhead_ns, predicted_kernels, device):
         self._total_ms = None
         self._overhead_ns = overhead_ns
         self._predicted_kernels, self._device = predicted_kernels, device
+        self._measured = self._times = None
 
-    kernels = _stored("_predicted_kernels")
+    @classmethod
+    def from_times(cls, overhead_ns, measured_kernels, times_ns, device):
+        self = cls(overhead_ns, None, device)
+        self._measured, self._times = measured_kernels, times_ns
+        return self
+
     device = _stored("_device")
+
+    @property
+    def kernels(self):
+        if self._predicted_kernels is None:
+            from habitat_amd.analysis.kernels import PredictedKernel
+            self._predicted_kernels = [PredictedKernel(k, t)
+                                       for k, t in zip(self._measured, self._times)]
+        return self._predicted_kernels
+
+    @property
+    def ktime_ns(self):
+        if self._predicted_kernels is None:
+            return sum(self._times)
+        return sum(kernel.run_time_ns for kernel in self._predicted_kernels)
 
     @property
     def run_time_ms(self):

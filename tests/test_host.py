@@ -312,3 +312,21 @@ def test_device_table_is_read_in_both_layouts(tmp_path, monkeypatch):
         assert table.names() == ["V100"]
         assert {f: getattr(table.V100, f) for f in v100} == v100
         assert table.V100.as_dict() == as_mapping
+
+
+def test_prediction_from_times_matches_one_from_kernels():
+    """A pass made from bare times reads like one made from PredictedKernels."""
+    from habitat_amd.analysis.kernels import KernelInstance, MeasuredKernel, PredictedKernel
+    from habitat_amd.analysis.run_time import RunTimePrediction
+    dev = Device.V100
+    measured = [MeasuredKernel(KernelInstance("k%d" % i, 10, 64, 0, 0, 32, 1000 + i), [], dev)
+                for i in range(3)]
+    times = [1500.25, 1001, 7.5]
+    lazy = RunTimePrediction.from_times(250.5, measured, times, dev)
+    eager = RunTimePrediction(250.5, [PredictedKernel(k, t) for k, t in zip(measured, times)], dev)
+    assert lazy.run_time_ms == eager.run_time_ms == (250.5 + 1500.25 + 1001 + 7.5) / 1e6
+    assert lazy.ktime_ns == eager.ktime_ns
+    assert [k.run_time_ns for k in lazy.kernels] == times
+    assert [k.name for k in lazy.kernels] == ["k0", "k1", "k2"]
+    assert lazy.kernels is lazy.kernels and lazy.ktime_ns == eager.ktime_ns
+    assert lazy.device is dev
