@@ -339,6 +339,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
+    from habitat_amd import _lib, build
+    if not os.path.exists(_lib.LIB_PATH):    # run what is built; compile only when nothing is
+        build.build()
     origin, dest = Device.V100, Device.MI355X
 
     if args.copy_calibration:

@@ -16,6 +16,16 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+@pytest.fixture(scope="session", autouse=True)
+def built_library():
+    """The tests load the library that is built; they compile it (hipcc
+    cross-compiles without a GPU) only when there is none."""
+    from habitat_amd import _lib, build
+    if not os.path.exists(_lib.LIB_PATH):
+        build.build()
+    return _lib.LIB_PATH
+
+
 @pytest.fixture(scope="session")
 def occupancy_golden():
     """(arrays, {device name: constructor kwargs}) written by
