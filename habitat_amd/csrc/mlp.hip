@@ -301,7 +301,11 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
 // The order of every sum is fixed, so results are reproducible.  Same packed
 // weights, same MFMA instruction, same fragment layout as above.
 constexpr int kSplit = 8;            // K-partials per hidden layer, up to kRows rows
-constexpr int kLayerMaxRows = 4096;  // largest batch that takes this path
+constexpr int kLayerMaxRows = 4096;  // largest batch that takes this path in one pass
+// Largest batch that takes this path in two passes (4096 rows, then the rest).
+// Measured, two passes against one round of the fused kernel (942 us): 4200
+// rows 702 us, 4608 755, 5120 808, 5686 954, 6144 965.
+constexpr int kLayerTwoPassRows = kLayerMaxRows + 1280;
 constexpr int kFewTiles = 8;         // m-tiles up to which the whole-K shape prefetches (DEPTH)
 constexpr int kManyTiles = 32;       // m-tiles from which its workgroups take four n-tiles (NT)
 constexpr size_t kScratchFloats = (size_t)kLayerMaxRows * kWidth;  // each of two buffers
@@ -834,19 +838,29 @@ int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* 
   if (device != mlp->device) return HBT_EINVAL;
 
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-  if (n <= kLayerMaxRows) return forward_layers(mlp, raw_features, n, out, stream);
   // The fused kernel keeps every compute unit busy for whole rounds of
-  // 32 rows x compute units (about 1 ms each); what is left over after the last
-  // whole round would cost another one.  Up to kLayerMaxRows leftover rows go
-  // through the per-layer path instead, which takes less.
+  // 32 rows x compute units (about 0.94 ms each); what is left over after the
+  // last whole round would cost another one.  Leftover rows go through the
+  // per-layer path instead where that takes less: up to kLayerMaxRows in one
+  // pass, up to kLayerTwoPassRows in two (the passes share the scratch buffers
+  // and follow each other on the stream).
   const int64_t round_rows = (int64_t)kRows * mlp->compute_units;
   const int64_t leftover = n % round_rows;
-  if (leftover == 0 || leftover > kLayerMaxRows)
+  if (leftover == 0 || leftover > kLayerTwoPassRows)
     return forward_fused(mlp, raw_features, n, out, stream);
-  const int64_t whole = n - leftover;
-  const int rc = forward_fused(mlp, raw_features, whole, out, stream);
-  if (rc != HBT_OK) return rc;
-  return forward_layers(mlp, raw_features + whole * mlp->in_features, leftover, out + whole, stream);
+  int64_t done = n - leftover;
+  if (done > 0) {
+    const int rc = forward_fused(mlp, raw_features, done, out, stream);
+    if (rc != HBT_OK) return rc;
+  }
+  while (done < n) {
+    const int64_t rows = n - done < kLayerMaxRows ? n - done : kLayerMaxRows;
+    const int rc = forward_layers(mlp, raw_features + done * mlp->in_features, rows, out + done,
+                                  stream);
+    if (rc != HBT_OK) return rc;
+    done += rows;
+  }
+  return HBT_OK;
 }
 
 void hbt_mlp_destroy(hbt_mlp* mlp) {
