@@ -36,6 +36,11 @@ def __getattr__(name):
         value = getattr(importlib.import_module(module), attr)
         globals()[name] = value
         return value
+    if name == "OperationTracker":
+        # analyzer/habitat/tracking/operation.py: measures operations with CUPTI on
+        # an NVIDIA GPU; it produces this path's input and is not part of it
+        raise AttributeError("habitat_amd has no OperationTracker: traces are measured with the "
+                             "reference's tracker and handed over as habitat_amd.analysis objects")
     raise AttributeError("module 'habitat_amd' has no attribute %r" % name)
 
 
