@@ -130,7 +130,7 @@ def tile_records(rec, n):
 
 def mlp_bench(args):
     """configs[2] (and the other kinds of configs[3], one step each): the fused
-    MLP at full size, the per-layer path (up to 5376 rows, 4096 at a time), and a torch CPU baseline."""
+    MLP at full size, the per-layer path (up to 6400 rows, 4096 at a time), and a torch CPU baseline."""
     import torch
     from habitat_amd import synthetic
     from habitat_amd.analysis.mlp.mlp import RuntimePredictor
@@ -185,7 +185,7 @@ def mlp_bench(args):
         for i in range(20):
             omlp.forward_fp32(sd, x[i:i + 1], mu, sigma)
         few["cpu_rows_1_us"] = (time.perf_counter() - t0) / 20 * 1e6
-    few["note"] = ("up to 5376 rows, 4096 at a time: one launch per layer over the whole GPU "
+    few["note"] = ("up to 6400 rows, 4096 at a time: one launch per layer over the whole GPU "
                    "(mlp_layer_kernel); "
                    "cpu_rows_1_us: torch CPU fp32, batch 1, as the reference predicts")
     mlp["few_rows"] = few

@@ -290,24 +290,28 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
 // K, each multiplies its k-groups straight from global memory (no loop, no LDS
 // staging) and the waves add their 32 x 32 accumulators through LDS.
 //
-//   33 rows and more: eight waves cover all of K (16 k-groups each), the
-//   workgroup applies bias and ReLU and writes activations, [row][n].
-//   Up to 32 rows that would be 32 workgroups per layer, so K is split kSplit
-//   ways over workgroups as well (four waves, 4 k-groups each) and the
+//   Otherwise eight waves cover all of K (16 k-groups each), the
+//   workgroup applies bias and ReLU and writes activations, stored by k-group
+//   (see km_index).
+//   For a few rows (up to kSplitMaxRows) K is split kSplit ways over
+//   workgroups as well (four waves, 4 k-groups each: 256 workgroups) and the
 //   K-partials are written as they are, [split][row][n]; they are summed,
 //   biased and rectified by whoever reads them: the next layer's activation
 //   load, or the final dot product.
 //
 // The order of every sum is fixed, so results are reproducible.  Same packed
 // weights, same MFMA instruction, same fragment layout as above.
-constexpr int kSplit = 8;            // K-partials per hidden layer, up to kRows rows
+constexpr int kSplit = 8;            // K-partials per hidden layer, up to kSplitMaxRows rows
+// Rows up to which K is split over workgroups.  Measured per forward at 1 / 8 /
+// 16 / 24 / 32 rows: split 39 44 52 61 71 us (the partials' traffic grows with
+// the rows), whole K 57 us at any of them.
+constexpr int kSplitMaxRows = 20;
 constexpr int kLayerMaxRows = 4096;  // largest batch that takes this path in one pass
 // Largest batch that takes this path in two passes (4096 rows, then the rest).
-// Measured, two passes against one round of the fused kernel (942 us): 4200
-// rows 702 us, 4608 755, 5120 808, 5686 954, 6144 965.
-constexpr int kLayerTwoPassRows = kLayerMaxRows + 1280;
-constexpr int kFewTiles = 8;         // m-tiles up to which the whole-K shape prefetches (DEPTH)
-constexpr int kManyTiles = 32;       // m-tiles from which its workgroups take four n-tiles (NT)
+// Measured, two passes against one round of the fused kernel (940 us): 4200
+// rows 612 us, 5120 712, 5686 841, 6144 846, 6656 913, 7168 979.
+constexpr int kLayerTwoPassRows = kLayerMaxRows + 2304;
+constexpr int kManyTiles = 32;       // m-tiles from which a workgroup takes two n-tiles (NT)
 constexpr size_t kScratchFloats = (size_t)kLayerMaxRows * kWidth;  // each of two buffers
 static_assert((size_t)kSplit * kRows * kWidth <= kScratchFloats, "the K-partials fit the scratch");
 
@@ -328,6 +332,15 @@ struct LayerArgs {
   int32_t m_pad;           // rows rounded up to 32
   float* p_out;            // [m_pad][kWidth] activations (FINAL), else [splits][m_pad][kWidth]
 };
+
+// Outside the split-K shape activations are stored by k-group (KM below): element
+// (row, n) at [row / 32][n / 8][row % 32][n % 8], so that the fragment a wave
+// loads for one m-tile and k-group, 32 rows x 8 values, is 1 KiB of contiguous
+// memory (8 cache lines used whole) where row-major storage spreads it over 32
+// lines, 32 bytes of each.
+__device__ __forceinline__ size_t km_index(int m_tile, int k_group, int m, int c) {
+  return (((size_t)m_tile * (kWidth / 8) + k_group) * kRows + m) * 8 + c;
+}
 
 // G k-groups of a wave: the weight fragments of the n-tile and what the
 // matching activation fragments are made from (the activations themselves, or
@@ -353,16 +366,26 @@ struct LayerFrag {
 //     the traffic of a handful of rows, not masking keeps the loads of a full
 //     tile free of branches.
 //   NT: n-tiles per workgroup (blockIdx.x counts groups of NT); an activation
-//     fragment then serves NT MFMAs.  Measured for the whole-K shape at 512 /
-//     1024 / 4096 rows: 1: 131 214 753 us; 2: 126 201 704; 4: 188 192 685.
+//     fragment then serves NT MFMAs.
 //   DEPTH: k-groups whose loads are kept in flight ahead of the MFMAs; 0 leaves
-//     the placement to the compiler.  Measured for the whole-K shape (us per
-//     forward at 64 / 256 / 512 / 4096 rows): 0: 80 88 132 766; 2: 70 77 137
-//     841; 4: 76 83 154 1014; 8: 90 97 188 1338; all 16: 95 102 178 1199.  More
-//     loads in flight only crowd the path from L2 once every compute unit has
-//     several workgroups; with a few m-tiles two groups ahead is best.
-template <bool FIRST, int S_IN, bool FINAL, int WAVES, bool PADDED_ROWS, int DEPTH, int NT = 1>
+//     the placement to the compiler (each group's loads next to its MFMAs, one
+//     trip to memory after the other, which resident workgroups hide from each
+//     other).
+//   KM: activations (read, unless FIRST, and written) are stored by k-group.
+// Measured for the whole-K shape with KM, us per forward at 256 / 512 / 768 /
+// 1024 / 1536 / 2048 / 4096 rows, as (DEPTH, NT):
+//   (0,1)  67 103 128 161 251 318 588     (0,2) 105 110 160 162 230 298 560
+//   (2,1)  67 103 130 160 274 319 596     (2,2)  95 100 154 154 280 291 605
+//   (4,1)  66 104 130 190 231 325 598     (0,4) 168 172 170 171 310 320 613
+//   (16,1) 71 116 154 194 277 360 693     (2,4) 157 161 158 159 287 299 567
+// so below 1024 rows a workgroup takes one n-tile with two groups in flight,
+// from there on two n-tiles and the compiler's placement.  (With row-major
+// activations, where a fragment touches 32 cache lines for 32 bytes each: 256
+// rows 74 us, 512 123, 1024 176 with four n-tiles, 4096 637.)
+template <bool FIRST, int S_IN, bool FINAL, int WAVES, bool PADDED_ROWS, int DEPTH, int NT = 1,
+          bool KM = false>
 __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a) {
+  static_assert(!KM || (S_IN == 0 && FINAL), "K-partials are row-major");
   static_assert(8 % NT == 0, "a workgroup's n-tiles lie in one wave stream of the packed weights");
   static_assert(S_IN == 0 || !FINAL, "K-partials go in and come out together");
   static_assert(WAVES == 4 || WAVES == 8, "the reduction below is written for these");
@@ -411,7 +434,8 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
                                                0x00020000);
     w_lane_bytes = ((tile & 7) * 64 + lane) * 16;
     w_base_bytes = ((tile >> 3) * a.groups_total + a.g0) * (8 * 64 * 16);
-    x_lane_bytes = row_ok ? (int)row * (kWidth * 4) + 16 * h : 0x7fffff00;
+    if (KM) x_lane_bytes = row_ok ? (int)km_index(blockIdx.z, 0, m, 4 * h) * 4 : 0x7fffff00;
+    else x_lane_bytes = row_ok ? (int)row * (kWidth * 4) + 16 * h : 0x7fffff00;
   }
   auto load_group = [&](int j) {
     if (!FIRST || j < count) {
@@ -424,7 +448,7 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
 #pragma unroll
         for (int s = 0; s < (S_IN > 0 ? S_IN : 1); ++s)
           f.x[j][s] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
-              x_rsrc, x_lane_bytes, s * split_bytes + gl * 32, 0));
+              x_rsrc, x_lane_bytes, s * split_bytes + gl * (KM ? kRows * 32 : 32), 0));
         if (S_IN > 0)
           f.bias[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
               b_rsrc, 16 * h, gl * 32, 0));
@@ -512,6 +536,7 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
       o[e] = sum;
     }
     float* dst = a.p_out + ((size_t)split * a.m_pad + (size_t)blockIdx.z * kRows + m) * kWidth + n0;
+    if (KM) dst = a.p_out + km_index(blockIdx.z, n0 >> 3, m, n0 & 7);
     if constexpr (R == 4) {
       *reinterpret_cast<f32x4*>(dst) = f32x4{o[0], o[1], o[2], o[3]};
     } else {
@@ -563,6 +588,34 @@ __global__ __launch_bounds__(256) void mlp_last_kernel(const LastArgs a) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off);
   if (lane == 0) a.out[row] = sum + a.b_last;
+}
+
+// fc2 from activations stored by k-group: one workgroup per m-tile, its four
+// waves take a quarter of K each; lane (m, h) reads 16 bytes of its row per
+// k-group, so that a wave's load is the k-group's contiguous 1 KiB.
+__global__ __launch_bounds__(256) void mlp_last_km_kernel(const LastArgs a) {
+  constexpr int kGroupsPerWave = kWidth / 8 / 4;
+  __shared__ float part[4][kRows];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int m = lane & 31, h = lane >> 5;
+  const f32x4* x = reinterpret_cast<const f32x4*>(
+      a.p_in + km_index(blockIdx.x, wave * kGroupsPerWave, m, 4 * h));
+  const f32x4* wl = reinterpret_cast<const f32x4*>(a.w_last + 8 * wave * kGroupsPerWave + 4 * h);
+  float sum = 0.f;
+#pragma unroll 8
+  for (int g = 0; g < kGroupsPerWave; ++g) {
+    const f32x4 v = x[(size_t)g * (kRows * 2)];
+    const f32x4 w = wl[2 * g];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum = fmaf(v[e], w[e], sum);
+  }
+  sum += __shfl_xor(sum, 32);
+  if (h == 0) part[wave][m] = sum;
+  __syncthreads();
+  const int64_t row = (int64_t)blockIdx.x * kRows + threadIdx.x;
+  if (threadIdx.x < kRows && row < a.n)
+    a.out[row] = ((part[0][threadIdx.x] + part[1][threadIdx.x]) +
+                  (part[2][threadIdx.x] + part[3][threadIdx.x])) + a.b_last;
 }
 
 constexpr int kWaves = 4;  // one wave per SIMD: measured faster than two (fewer, longer MFMA runs between load bursts)
@@ -622,7 +675,7 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
   using namespace hbt;
   // one launch per layer, through the handle's two scratch buffers
   const int m_tiles = (int)((n + kRows - 1) / kRows);
-  const bool split_k = m_tiles == 1;
+  const bool split_k = n <= kSplitMaxRows;
   LayerArgs l{};
   l.w_stream = mlp->w_stream;
   l.groups_total = mlp->in_padded / 8 + mlp->hidden * (kWidth / 8);
@@ -641,18 +694,18 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
     l.bias_out = mlp->bias + (size_t)layer * kWidth;
     l.p_out = mlp->scratch[layer & 1];
     const dim3 grid(kWidth / 32, (unsigned)l.splits, (unsigned)m_tiles);
-    if (layer == 0)
+    if (layer == 0 && split_k)
       hipLaunchKernelGGL((mlp_layer_kernel<true, 0, true, 4, false, 0>), grid, dim3(256), 0,
                          stream, l);
-    else if (!split_k && m_tiles <= kFewTiles)
-      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 2>), grid, dim3(512), 0,
-                         stream, l);
-    else if (!split_k && m_tiles >= kManyTiles)
-      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 0, 4>),
-                         dim3(kWidth / 128, 1, (unsigned)m_tiles), dim3(512), 0, stream, l);
+    else if (layer == 0)
+      hipLaunchKernelGGL((mlp_layer_kernel<true, 0, true, 4, false, 0, 1, true>), grid, dim3(256),
+                         0, stream, l);
+    else if (!split_k && m_tiles < kManyTiles)
+      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 2, 1, true>), grid, dim3(512),
+                         0, stream, l);
     else if (!split_k)
-      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 0>), grid, dim3(512), 0,
-                         stream, l);
+      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 0, 2, true>),
+                         dim3(kWidth / 64, 1, (unsigned)m_tiles), dim3(512), 0, stream, l);
     else if (partials)
       hipLaunchKernelGGL((mlp_layer_kernel<false, kSplit, false, 4, false, 0>), grid, dim3(256),
                          0, stream, l);
@@ -669,7 +722,8 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
   z.n = n; z.m_pad = l.m_pad; z.out = out;
   const dim3 rows_grid((unsigned)((n + 3) / 4));
   if (partials) hipLaunchKernelGGL(mlp_last_kernel<kSplit>, rows_grid, dim3(256), 0, stream, z);
-  else hipLaunchKernelGGL(mlp_last_kernel<0>, rows_grid, dim3(256), 0, stream, z);
+  else if (split_k) hipLaunchKernelGGL(mlp_last_kernel<0>, rows_grid, dim3(256), 0, stream, z);
+  else hipLaunchKernelGGL(mlp_last_km_kernel, dim3((unsigned)m_tiles), dim3(256), 0, stream, z);
   return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
 }
 
