@@ -292,7 +292,8 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
 //
 //   Otherwise eight waves cover all of K (16 k-groups each), the
 //   workgroup applies bias and ReLU and writes activations, stored by k-group
-//   (see km_index).
+//   (see km_index).  Up to kHalfKMaxTiles m-tiles K is split over two such
+//   workgroups, whose K-partials are stored the same way.
 //   For a few rows (up to kSplitMaxRows) K is split kSplit ways over
 //   workgroups as well (four waves, 4 k-groups each: 256 workgroups) and the
 //   K-partials are written as they are, [split][row][n]; they are summed,
@@ -312,6 +313,11 @@ constexpr int kLayerMaxRows = 4096;  // largest batch that takes this path in on
 // rows 612 us, 5120 712, 5686 841, 6144 846, 6656 913, 7168 979.
 constexpr int kLayerTwoPassRows = kLayerMaxRows + 2304;
 constexpr int kManyTiles = 32;       // m-tiles from which a workgroup takes two n-tiles (NT)
+// m-tiles up to which the eight-wave shape splits K over two workgroups (128
+// workgroups or fewer per layer would leave half the compute units idle).
+// Measured per forward at 32 / 64 / 128 / 256 rows: 49 52 58 82 us against 57 57
+// 59 65 without; four K-partials were no faster than two.
+constexpr int kHalfKMaxTiles = 4;
 constexpr size_t kScratchFloats = (size_t)kLayerMaxRows * kWidth;  // each of two buffers
 static_assert((size_t)kSplit * kRows * kWidth <= kScratchFloats, "the K-partials fit the scratch");
 
@@ -321,7 +327,7 @@ struct LayerArgs {
   int32_t g0;              // first stream group of this layer
   int32_t kg;              // k-groups of this layer (K / 8)
   int32_t splits;          // K-partials this launch writes (gridDim.y)
-  const float* p_in;       // [m_pad][kWidth] activations, or [kSplit][m_pad][kWidth] partials
+  const float* p_in;       // m_pad x kWidth activations, or S_IN such blocks of K-partials
   const float* bias_in;    // [kWidth], bias of the previous layer (with partials)
   const float* bias_out;   // [kWidth], bias of this layer (FINAL)
   const double* raw;       // FIRST: [n][in_features], with mu and sigma
@@ -330,7 +336,7 @@ struct LayerArgs {
   int32_t in_features;
   int64_t n;
   int32_t m_pad;           // rows rounded up to 32
-  float* p_out;            // [m_pad][kWidth] activations (FINAL), else [splits][m_pad][kWidth]
+  float* p_out;            // m_pad x kWidth activations (FINAL), else `splits` blocks of partials
 };
 
 // Outside the split-K shape activations are stored by k-group (KM below): element
@@ -357,7 +363,7 @@ struct LayerFrag {
 // k-groups (at most G each); fc1 has fewer, so there each group is checked
 // against the wave's count (wave-uniform).
 //   FIRST: fc1, from the raw fp64 rows, standardised on the spot.
-//   S_IN: 0 = the input holds activations; kSplit = it holds that many
+//   S_IN: 0 = the input holds activations; otherwise it holds that many
 //     K-partials, to be summed, biased and rectified on the way in.
 //   FINAL: the launch covers all of K (a.splits == 1), so the output is
 //     biased and rectified here and the next layer reads activations.
@@ -382,14 +388,15 @@ struct LayerFrag {
 // from there on two n-tiles and the compiler's placement.  (With row-major
 // activations, where a fragment touches 32 cache lines for 32 bytes each: 256
 // rows 74 us, 512 123, 1024 176 with four n-tiles, 4096 637.)
+//   S_OUT: K-partials this launch writes (a.splits; 1 with FINAL).
 template <bool FIRST, int S_IN, bool FINAL, int WAVES, bool PADDED_ROWS, int DEPTH, int NT = 1,
-          bool KM = false>
+          bool KM = false, int S_OUT = (FINAL ? 1 : kSplit)>
 __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a) {
-  static_assert(!KM || (S_IN == 0 && FINAL), "K-partials are row-major");
+  static_assert((S_OUT == 1) == FINAL, "one K-partial is the whole sum");
   static_assert(8 % NT == 0, "a workgroup's n-tiles lie in one wave stream of the packed weights");
   static_assert(S_IN == 0 || !FINAL, "K-partials go in and come out together");
   static_assert(WAVES == 4 || WAVES == 8, "the reduction below is written for these");
-  constexpr int G = FIRST ? kMaxInPadded / 8 / WAVES : kWidth / 8 / WAVES / (FINAL ? 1 : kSplit);
+  constexpr int G = FIRST ? kMaxInPadded / 8 / WAVES : kWidth / 8 / WAVES / S_OUT;
   __shared__ float red[WAVES][NT][16][64];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -536,7 +543,8 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
       o[e] = sum;
     }
     float* dst = a.p_out + ((size_t)split * a.m_pad + (size_t)blockIdx.z * kRows + m) * kWidth + n0;
-    if (KM) dst = a.p_out + km_index(blockIdx.z, n0 >> 3, m, n0 & 7);
+    if (KM)
+      dst = a.p_out + (size_t)split * a.m_pad * kWidth + km_index(blockIdx.z, n0 >> 3, m, n0 & 7);
     if constexpr (R == 4) {
       *reinterpret_cast<f32x4*>(dst) = f32x4{o[0], o[1], o[2], o[3]};
     } else {
@@ -546,7 +554,7 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
 }
 
 struct LastArgs {
-  const float* p_in;     // [m_pad][kWidth] activations, or [kSplit][m_pad][kWidth] partials
+  const float* p_in;     // m_pad x kWidth activations, or S_IN such blocks of K-partials
   const float* bias_in;  // [kWidth], bias of the last hidden layer (with partials)
   const float* w_last;   // [kWidth]
   float b_last;
@@ -593,6 +601,7 @@ __global__ __launch_bounds__(256) void mlp_last_kernel(const LastArgs a) {
 // fc2 from activations stored by k-group: one workgroup per m-tile, its four
 // waves take a quarter of K each; lane (m, h) reads 16 bytes of its row per
 // k-group, so that a wave's load is the k-group's contiguous 1 KiB.
+template <int S_IN>
 __global__ __launch_bounds__(256) void mlp_last_km_kernel(const LastArgs a) {
   constexpr int kGroupsPerWave = kWidth / 8 / 4;
   __shared__ float part[4][kRows];
@@ -601,13 +610,36 @@ __global__ __launch_bounds__(256) void mlp_last_km_kernel(const LastArgs a) {
   const f32x4* x = reinterpret_cast<const f32x4*>(
       a.p_in + km_index(blockIdx.x, wave * kGroupsPerWave, m, 4 * h));
   const f32x4* wl = reinterpret_cast<const f32x4*>(a.w_last + 8 * wave * kGroupsPerWave + 4 * h);
+  constexpr int P = S_IN > 0 ? S_IN : 1;
+  constexpr int kStep = 8;  // k-groups whose loads are issued together
   float sum = 0.f;
-#pragma unroll 8
-  for (int g = 0; g < kGroupsPerWave; ++g) {
-    const f32x4 v = x[(size_t)g * (kRows * 2)];
-    const f32x4 w = wl[2 * g];
+  for (int g0 = 0; g0 < kGroupsPerWave; g0 += kStep) {
+    f32x4 v[kStep][P], w[kStep], bias[kStep];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) sum = fmaf(v[e], w[e], sum);
+    for (int j = 0; j < kStep; ++j) {
+#pragma unroll
+      for (int s = 0; s < P; ++s)
+        v[j][s] = x[(size_t)(g0 + j) * (kRows * 2) + (size_t)s * a.m_pad * (kWidth / 4)];
+      w[j] = wl[2 * (g0 + j)];
+      if (S_IN > 0)
+        bias[j] = *reinterpret_cast<const f32x4*>(
+            a.bias_in + 8 * (wave * kGroupsPerWave + g0 + j) + 4 * h);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // all of the step's loads before its arithmetic
+#pragma unroll
+    for (int j = 0; j < kStep; ++j) {
+      f32x4 act = v[j][0];
+      if (S_IN > 0) {
+        // K-partials in their fixed order, then bias and ReLU
+        act = bias[j];
+#pragma unroll
+        for (int s = 0; s < S_IN; ++s) act += v[j][s];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) act[e] = relu(act[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sum = fmaf(act[e], w[j][e], sum);
+    }
   }
   sum += __shfl_xor(sum, 32);
   if (h == 0) part[wave][m] = sum;
@@ -676,6 +708,8 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
   // one launch per layer, through the handle's two scratch buffers
   const int m_tiles = (int)((n + kRows - 1) / kRows);
   const bool split_k = n <= kSplitMaxRows;
+  // with a few m-tiles the eight-wave shape splits K in two as well
+  const int ks = (!split_k && m_tiles <= kHalfKMaxTiles) ? 2 : 1;
   LayerArgs l{};
   l.w_stream = mlp->w_stream;
   l.groups_total = mlp->in_padded / 8 + mlp->hidden * (kWidth / 8);
@@ -688,7 +722,7 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
   for (int layer = 0; layer <= mlp->hidden; ++layer) {
     l.g0 = (layer == 0) ? 0 : mlp->in_padded / 8 + (layer - 1) * (kWidth / 8);
     l.kg = (layer == 0) ? mlp->in_padded / 8 : kWidth / 8;
-    l.splits = (layer > 0 && split_k) ? kSplit : 1;
+    l.splits = layer == 0 ? 1 : (split_k ? kSplit : ks);
     l.p_in = p_in;
     l.bias_in = (layer == 0) ? nullptr : mlp->bias + (size_t)(layer - 1) * kWidth;
     l.bias_out = mlp->bias + (size_t)layer * kWidth;
@@ -700,6 +734,12 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
     else if (layer == 0)
       hipLaunchKernelGGL((mlp_layer_kernel<true, 0, true, 4, false, 0, 1, true>), grid, dim3(256),
                          0, stream, l);
+    else if (ks == 2 && !partials)
+      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, false, 8, true, 2, 1, true, 2>), grid,
+                         dim3(512), 0, stream, l);
+    else if (ks == 2)
+      hipLaunchKernelGGL((mlp_layer_kernel<false, 2, false, 8, true, 2, 1, true, 2>), grid,
+                         dim3(512), 0, stream, l);
     else if (!split_k && m_tiles < kManyTiles)
       hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 2, 1, true>), grid, dim3(512),
                          0, stream, l);
@@ -721,9 +761,12 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
   z.w_last = mlp->w_last; z.b_last = mlp->b_last;
   z.n = n; z.m_pad = l.m_pad; z.out = out;
   const dim3 rows_grid((unsigned)((n + 3) / 4));
-  if (partials) hipLaunchKernelGGL(mlp_last_kernel<kSplit>, rows_grid, dim3(256), 0, stream, z);
+  if (partials && split_k)
+    hipLaunchKernelGGL(mlp_last_kernel<kSplit>, rows_grid, dim3(256), 0, stream, z);
   else if (split_k) hipLaunchKernelGGL(mlp_last_kernel<0>, rows_grid, dim3(256), 0, stream, z);
-  else hipLaunchKernelGGL(mlp_last_km_kernel, dim3((unsigned)m_tiles), dim3(256), 0, stream, z);
+  else if (partials && ks == 2)
+    hipLaunchKernelGGL(mlp_last_km_kernel<2>, dim3((unsigned)m_tiles), dim3(256), 0, stream, z);
+  else hipLaunchKernelGGL(mlp_last_km_kernel<0>, dim3((unsigned)m_tiles), dim3(256), 0, stream, z);
   return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
 }
 

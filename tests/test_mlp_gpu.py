@@ -114,7 +114,7 @@ def test_the_three_paths_agree_on_the_same_rows():
 
 
 @pytest.mark.parametrize("hidden", [0, 1, 3])
-@pytest.mark.parametrize("rows", [5, 130, 4200, 6500])
+@pytest.mark.parametrize("rows", [5, 40, 130, 4200, 6500])
 def test_other_depths(hidden, rows):
     """Networks with no, one and three hidden layers through all three paths
     (the kernels take the depth from the handle; without hidden layers the final
