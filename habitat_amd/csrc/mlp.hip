@@ -280,25 +280,26 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
 
 // ---------------------------------------------------------------------------
 // Up to a few thousand rows (one prediction, the operations of one trace, a
-// trace for a handful of devices): one launch per layer.
+// trace for some devices): one launch per layer.
 //
 // The fused kernel gives each workgroup 32 rows and the whole network, so a
 // batch of up to 32 rows runs on ONE compute unit, which has to pull all
 // 33.6 MB of weights through by itself (about 1 ms), and any batch below 8192
 // rows leaves compute units idle for that long.  Here a layer is spread over
-// the chip instead: a workgroup takes one n-tile x one m-tile, its waves split
-// K, each multiplies its k-groups straight from global memory (no loop, no LDS
-// staging) and the waves add their 32 x 32 accumulators through LDS.
+// the chip instead: a workgroup takes one or two n-tiles x one m-tile, its
+// waves split K, each multiplies its k-groups straight from global memory (no
+// loop, no LDS staging) and the waves add their 32 x 32 accumulators through
+// LDS.
 //
-//   Otherwise eight waves cover all of K (16 k-groups each), the
-//   workgroup applies bias and ReLU and writes activations, stored by k-group
-//   (see km_index).  Up to kHalfKMaxTiles m-tiles K is split over two such
-//   workgroups, whose K-partials are stored the same way.
 //   For a few rows (up to kSplitMaxRows) K is split kSplit ways over
 //   workgroups as well (four waves, 4 k-groups each: 256 workgroups) and the
 //   K-partials are written as they are, [split][row][n]; they are summed,
 //   biased and rectified by whoever reads them: the next layer's activation
 //   load, or the final dot product.
+//   Otherwise eight waves cover all of K (16 k-groups each), the workgroup
+//   applies bias and ReLU and writes activations, stored by k-group (see
+//   km_index).  Up to kHalfKMaxTiles m-tiles K is split over two such
+//   workgroups, whose K-partials are stored by k-group too.
 //
 // The order of every sum is fixed, so results are reproducible.  Same packed
 // weights, same MFMA instruction, same fragment layout as above.
@@ -378,6 +379,7 @@ struct LayerFrag {
 //     trip to memory after the other, which resident workgroups hide from each
 //     other).
 //   KM: activations (read, unless FIRST, and written) are stored by k-group.
+//   S_OUT: K-partials this launch writes (a.splits; 1 with FINAL).
 // Measured for the whole-K shape with KM, us per forward at 256 / 512 / 768 /
 // 1024 / 1536 / 2048 / 4096 rows, as (DEPTH, NT):
 //   (0,1)  67 103 128 161 251 318 588     (0,2) 105 110 160 162 230 298 560
@@ -388,7 +390,6 @@ struct LayerFrag {
 // from there on two n-tiles and the compiler's placement.  (With row-major
 // activations, where a fragment touches 32 cache lines for 32 bytes each: 256
 // rows 74 us, 512 123, 1024 176 with four n-tiles, 4096 637.)
-//   S_OUT: K-partials this launch writes (a.splits; 1 with FINAL).
 template <bool FIRST, int S_IN, bool FINAL, int WAVES, bool PADDED_ROWS, int DEPTH, int NT = 1,
           bool KM = false, int S_OUT = (FINAL ? 1 : kSplit)>
 __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a) {
