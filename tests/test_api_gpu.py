@@ -228,6 +228,40 @@ def test_device_sweep_matches_per_device_prediction():
         assert md.DEVICE_FEATURES == before
 
 
+def test_odd_traces_through_both_interfaces():
+    """Traces without operations, without kernels, without MLP-predicted
+    operations, without wave-scaled ones or without backward passes: per device
+    (`to_device`) and as a sweep (`to_devices`) give the same totals."""
+    from habitat_amd.analysis.operation import MeasuredOperation
+    from habitat_amd.analysis.run_time import RunTimeMeasurement
+    origin = Device.V100
+    ops = synthetic.resnet50_trace(origin, batch=32, seed=3).operations
+    predictor = Predictor(mlp_predictors=seeded_predictors())
+    scaled = [o for o in ops if o.name not in ("conv2d", "linear")]
+    mlp = [o for o in ops if o.name in ("conv2d", "linear")]
+    no_backward = [MeasuredOperation(o.name, o.arguments, o.forward, None, o.device)
+                   for o in scaled[:7]]
+    no_kernels = [MeasuredOperation("relu", scaled[0].arguments,
+                                    RunTimeMeasurement(0.25, [], origin), None, origin)]
+    dests = [Device.T4, Device.P100, Device.RTX2070]
+    cases = {"empty": [], "wave-scaled only": scaled, "mlp only": mlp, "no backward": no_backward,
+             "no kernels": no_kernels, "one operation": scaled[:1], "one mlp operation": mlp[:1],
+             "mixed": scaled[:3] + mlp[:2] + no_kernels}
+    for name, case in cases.items():
+        trace = Trace(origin, list(case))
+        one_by_one = [trace.to_device(d, predictor).run_time_ms for d in dests]
+        swept = trace.to_devices(dests, predictor)
+        assert len(swept) == 3, name
+        assert np.allclose(one_by_one, swept, rtol=1e-6, atol=1e-12), name
+        if name == "empty":
+            assert one_by_one == [0, 0, 0]
+        if name == "no kernels":
+            assert one_by_one == [0.25] * 3      # nothing to scale: the overhead alone
+        if name == "no backward":
+            want = opred.trace_ms([oracle_operation_ms(op, dests[0], {}) for op in case])
+            assert one_by_one[0] == pytest.approx(want, rel=1e-6)
+
+
 def test_local_device_description_and_measured_ceilings():
     from habitat_amd import device_info
     name, props = device_info.local_device(0)
