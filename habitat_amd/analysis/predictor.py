@@ -191,6 +191,12 @@ class Predictor:
                 logger.warning("Unhandled special operation: %s", op.name)
                 results[i] = PredictedOperation(op, op.forward, op.backward, dest_device)
 
+        # The MLP launches go first and are read back last, so that the GPU runs
+        # them while the host assembles the wave-scaled passes.
+        pending = [(idxs, [operations[i] for i in idxs]) for idxs in special.values()]
+        pending = [(idxs, ops, self._special_enqueue(ops[0].name, ops, dest_device))
+                   for idxs, ops in pending]
+
         if scaled:
             passes = []  # (op index, is_backward, run_time)
             for i in scaled:
@@ -205,9 +211,8 @@ class Predictor:
             for i in scaled:
                 results[i] = PredictedOperation(operations[i], fwd[i], bwd.get(i), dest_device)
 
-        for kind, idxs in special.items():
-            ops = [operations[i] for i in idxs]
-            for i, ms in zip(idxs, self._special_scale_many(kind, ops, dest_device)):
+        for idxs, ops, y in pending:
+            for i, ms in zip(idxs, self._special_finish(ops, y)):
                 results[i] = PredictedOperation(
                     operations[i], RunTimePurePrediction(ms, dest_device), None, dest_device)
         return results
@@ -298,6 +303,13 @@ class Predictor:
     def _special_scale_many(self, kind, operations, dest_device):
         """predictor.py:132-148 and the four scalers (:150-283), batched: one MLP
         launch evaluates every operation on its origin and on the destination."""
+        return self._special_finish(operations,
+                                    self._special_enqueue(kind, operations, dest_device))
+
+    def _special_enqueue(self, kind, operations, dest_device):
+        """The MLP launch of _special_scale_many; returns its output, still on
+        the GPU: rows 2i and 2i+1 are operation i on the destination and on its
+        origin."""
         pred = self._mlp(kind)
         rows = []
         dest_feats = get_device_features(dest_device.name, pred.device_params)
@@ -306,7 +318,13 @@ class Predictor:
             feats = [a[x] for x in pred.model.features]
             rows.append(feats + dest_feats)
             rows.append(feats + get_device_features(op.device.name, pred.device_params))
-        y = pred.predict_batch(np.asarray(rows, np.float64)).cpu().numpy().astype(np.float64)
+        return pred.predict_batch(np.asarray(rows, np.float64))
+
+    @staticmethod
+    def _special_finish(operations, y):
+        """Measured time x predicted destination time / predicted origin time,
+        not below zero (predictor.py:132-148)."""
+        y = y.cpu().numpy().astype(np.float64)
         out = []
         for i, op in enumerate(operations):
             ms = op.run_time_ms * float(y[2 * i]) / float(y[2 * i + 1])
