@@ -5,10 +5,11 @@ Same three classes and read-only attributes as the reference
 `backward`, `device`, the sums `run_time_ms` and `ktime_ns` over the passes an
 operation has, and `to_device`.
 """
+import operator
 
 
 def _read_only(slot):
-    return property(lambda self: getattr(self, slot))
+    return property(operator.attrgetter(slot))
 
 
 def _abstract(self):

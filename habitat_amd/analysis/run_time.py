@@ -2,6 +2,7 @@
 predicted from kernels, or predicted outright.  Same four classes and read-only
 attributes as the reference (analyzer/habitat/analysis/run_time.py:5-88):
 `run_time_ms`, `kernels`, `device` and the kernel-time sum `ktime_ns`."""
+import operator
 
 
 def ns_to_ms(ns):
@@ -13,7 +14,7 @@ def ms_to_ns(ms):
 
 
 def _stored(slot):
-    return property(lambda self: getattr(self, slot))
+    return property(operator.attrgetter(slot))
 
 
 def _missing(self):
