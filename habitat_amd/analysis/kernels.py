@@ -50,6 +50,12 @@ class KernelInstance:
             "registers_per_thread": self._registers_per_thread,
         }
 
+    def launch_fields(self):
+        """(num_blocks, block_size, dynamic_smem, static_smem, regs, run_time_ns):
+        what `metadata`, `num_blocks` and `run_time_ns` hold, without the dict."""
+        return (self._num_blocks, self._block_size, self._dynamic_shared_memory,
+                self._static_shared_memory, self._registers_per_thread, self._run_time_ns)
+
     def thread_block_occupancy(self, device, registers_per_thread=-1):
         """Blocks per multiprocessor on `device`; a negative register count
         means this kernel's own (model_bindings.cpp:75-82)."""
@@ -78,6 +84,15 @@ class MeasuredKernel:
         if default is None:
             raise AttributeError("Unknown metric: {}".format(metric_info.name))
         return default
+
+    # the attributes read per kernel on the prediction path, without the detour
+    # through __getattr__
+    name = property(lambda self: self._c.name)
+    run_time_ns = property(lambda self: self._c.run_time_ns)
+    num_blocks = property(lambda self: self._c.num_blocks)
+
+    def launch_fields(self):
+        return self._c.launch_fields()
 
     def __getattr__(self, name):
         # Everything else comes from the underlying kernel instance.

@@ -113,20 +113,21 @@ def occupancy_device(device, mode):
 def records_from_kernels(kernels, dest_device, metadata_manager, mode="unified", device=None):
     """Python kernel objects -> KernelRecords on the GPU (one upload)."""
     n = len(kernels)
-    ints = np.empty((5, n), np.int32)
-    f64 = np.zeros((4, n), np.float64)
-    has = np.zeros(n, np.uint8)
-    for i, k in enumerate(kernels):
-        nb, block, dyn, stat, regs, t_ns = kernel_fields(k)
-        ints[:, i] = (nb, block, dyn, stat, regs)
-        f64[0, i] = t_ns
-        if mode != "resimplified":
+    fields = list(zip(*[kernel_fields(k) for k in kernels])) if n else [()] * 6
+    metrics = [(0.0, 0.0, 0.0)] * n
+    has = [0] * n
+    if mode != "resimplified":
+        for i, k in enumerate(kernels):
             try:
-                f64[1:, i] = [k.get_metric(m) for m in _METRICS]
+                metrics[i] = [k.get_metric(m) for m in _METRICS]
                 has[i] = 1
             except AttributeError:
                 if mode == "roofline":
                     raise
+    ints = [np.array(fields[j], np.int32) for j in range(5)]
+    f64 = [np.array(fields[5], np.float64)] + [
+        np.array(col, np.float64) for col in (zip(*metrics) if n else [(), (), ()])]
+    has = np.array(has, np.uint8)
     if hasattr(metadata_manager, "registers_for_names"):
         dest_regs = metadata_manager.registers_for_names([k.name for k in kernels], dest_device)
     else:
