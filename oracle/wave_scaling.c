@@ -22,8 +22,11 @@
  *
  * pins: tests/test_oracle.py checks this file against oracle/wave_scaling.py
  * (a line-by-line Python restatement), against the hand-derived known answers
- * of tests/golden/scaling_kat.json and against closed forms (identity, gamma
- * 0 and 1, continuity at the ridge point).
+ * of tests/golden/kat.json (both branches of gamma, below and above the ridge
+ * point; the small-kernel factor with unequal ceilings on the two devices;
+ * table registers that move a record from one branch to the other; the
+ * no-metrics strategy on both branches) and against closed forms (identity,
+ * gamma 0 and 1, continuity at the ridge point).
  */
 #include <math.h>
 #include <stddef.h>

@@ -15,7 +15,9 @@ A record is a mapping with the keys of `KEYS`; a device is an oracle.lib.Device.
 `occupancy` is injected so that tests can run this file over either the
 oracle's C routine or the compiled reference routine.
 
-pins: the three hand-derived known answers in tests/golden/scaling_kat.json;
+pins: the hand-derived known answers in tests/golden/kat.json (gamma below and
+above the ridge point, the small-kernel factor with ceilings 2 and 3, 4 and 6,
+a register-table entry that changes the branch, the no-metrics strategy);
 closed forms (same device both sides is the identity; flop efficiency 0 gives
 t*bw_o/bw_d; zero bytes give t*(clk_o/clk_d)*(sms_o/sms_d); intensity equal to
 the ridge point gives gamma 0.5 from either side).

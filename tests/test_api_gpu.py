@@ -63,11 +63,19 @@ def test_scalar_strategies_known_answers(kat):
     mm = NullMetadataManager()
     for row in kat["scaling"]:
         o, d = getattr(Device, row["origin"]), getattr(Device, row["dest"])
-        k = make_kernel(o, num_blocks=row["num_blocks"])
-        for strategy in (unified_wave_scaling, roofline_wave_scaling):
-            p = strategy(k, o, d, mm)
+        over = row.get("record", {})
+        metrics = (over.get("flop_sp_efficiency", 50.0), 1e8, 1e8)
+        has_metrics = row.get("has_metrics", True)
+        k = make_kernel(o, num_blocks=row["num_blocks"], metrics=metrics if has_metrics else None)
+        manager = mm if "dest_regs" not in row else TableManager({("k", d.name): row["dest_regs"]})
+        strategies = (unified_wave_scaling, roofline_wave_scaling) if has_metrics else (
+            unified_wave_scaling, resimplified_wave_scaling)
+        for strategy in strategies:
+            p = strategy(k, o, d, manager)
             assert isinstance(p, PredictedKernel) and p.name == "k"
             assert p.run_time_ns == pytest.approx(row["time_ns"], rel=1e-6)
+        if "occ_dest" in row:
+            assert k.thread_block_occupancy(d, row.get("dest_regs", -1)) == row["occ_dest"]
     # no metrics: unified falls back, roofline raises AttributeError like the reference
     k = make_kernel(Device.V100, metrics=None)
     assert unified_wave_scaling(k, Device.V100, Device.P100, mm).run_time_ns == pytest.approx(

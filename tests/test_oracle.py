@@ -93,17 +93,37 @@ def _cols(recs):
     return {k: np.array([r[k] for r in recs]) for k in recs[0]}
 
 
+def _kat_case(kat, row):
+    """(record, origin, dest, dest_regs, has_metrics) of one scaling known answer."""
+    o, d = oracle_device(DEVS[row["origin"]]), oracle_device(DEVS[row["dest"]])
+    rec = _record(kat, row["num_blocks"], **row.get("record", {}))
+    return rec, o, d, row.get("dest_regs"), row.get("has_metrics", True)
+
+
 def test_scaling_known_answers_python_and_c(kat):
+    assert sum(r.get("above_ridge", False) for r in kat["scaling"]) >= 3
+    assert any(r.get("origin_ceiling", 0) != r.get("dest_ceiling", 0) for r in kat["scaling"])
     for row in kat["scaling"]:
-        o, d = oracle_device(DEVS[row["origin"]]), oracle_device(DEVS[row["dest"]])
-        rec = _record(kat, row["num_blocks"])
-        assert ows.gamma(rec, o, d) == pytest.approx(row["gamma"], rel=1e-15)
-        assert ows.unified(rec, o, d) == pytest.approx(row["time_ns"], rel=1e-14)
-        c = olib.wave_scale(o, d, _cols([rec]), want_gamma=True)
+        rec, o, d, dest_regs, hm = _kat_case(kat, row)
+        if hm:
+            assert ows.gamma(rec, o, d) == pytest.approx(row["gamma"], rel=1e-15)
+        assert ows.unified(rec, o, d, dest_regs, hm) == pytest.approx(row["time_ns"], rel=1e-14)
+        cols = _cols([rec])
+        cols["has_metrics"] = np.array([hm], np.uint8)
+        if dest_regs is not None:
+            cols["dest_regs"] = np.array([dest_regs], np.int32)
+        c = olib.wave_scale(o, d, cols, want_gamma=True)
         assert c["status"][0] == 0
         assert c["time_ns"][0] == pytest.approx(row["time_ns"], rel=1e-14)
-        assert c["gamma"][0] == pytest.approx(row["gamma"], rel=1e-15)
-        wave_o, wave_d, _, _ = ows.wave_info(rec, o, d)
+        if hm:
+            assert c["gamma"][0] == pytest.approx(row["gamma"], rel=1e-15)
+        wave_o, wave_d, occ_o, occ_d = ows.wave_info(rec, o, d, dest_regs)
+        for key, got, got_c in (("occ_origin", occ_o, c["occ_origin"][0]),
+                                ("occ_dest", occ_d, c["occ_dest"][0]),
+                                ("wave_origin", wave_o, c["wave_origin"][0]),
+                                ("wave_dest", wave_d, c["wave_dest"][0])):
+            if key in row:
+                assert got == row[key] == got_c, (key, row)
         small = row["num_blocks"] < wave_o and row["num_blocks"] < wave_d
         assert small == (row["branch"] == "small")
 
@@ -242,9 +262,9 @@ def test_python_restatement_over_compiled_reference_occupancy(kat):
         return int(ref.ref_occupancy(ctypes.byref(dev), rec["block_size"], rec["dynamic_smem"],
                                      rec["static_smem"], rec["regs_per_thread"], regs))
     for row in kat["scaling"]:
-        o, d = oracle_device(DEVS[row["origin"]]), oracle_device(DEVS[row["dest"]])
-        rec = _record(kat, row["num_blocks"])
-        assert ows.unified(rec, o, d, occupancy=ref_occ) == pytest.approx(row["time_ns"], rel=1e-14)
+        rec, o, d, dest_regs, hm = _kat_case(kat, row)
+        assert ows.unified(rec, o, d, dest_regs, hm, occupancy=ref_occ) == pytest.approx(
+            row["time_ns"], rel=1e-14)
 
 
 def test_predictor_arithmetic():

@@ -61,6 +61,43 @@ def test_config1_1m_records():
     assert bool(torch.all(t < torch.from_numpy(rec["run_time_ns"]).cuda()))
 
 
+def test_hand_worked_known_answers_through_the_batch_kernel(kat):
+    """The kernel against the numbers worked by hand from roofline.py:8-104 and
+    resimplified.py:7-40 (tests/golden/kat.json), without the oracle in between:
+    gamma above and below the ridge point, unequal small-kernel ceilings, a
+    register-table entry that changes the branch, records without metrics.
+    All rows of one (origin, destination) pair go through one launch."""
+    pairs = {}
+    for row in kat["scaling"]:
+        pairs.setdefault((row["origin"], row["dest"]), []).append(row)
+    for (oname, dname), rows in pairs.items():
+        recs = [dict(kat["scaling_record"], num_blocks=r["num_blocks"], **r.get("record", {}))
+                for r in rows]
+        rec = {k: np.array([r[k] for r in recs]) for k in recs[0]}
+        rec = {k: v.astype(np.float64 if k in ("run_time_ns", "flop_sp_efficiency", "dram_read_bytes",
+                                                "dram_write_bytes") else np.int32)
+               for k, v in rec.items()}
+        rec["dest_regs"] = np.array([r.get("dest_regs", -1) for r in rows], np.int32)
+        rec["has_metrics"] = np.array([r.get("has_metrics", True) for r in rows], np.uint8)
+        out = wave_scale(KernelRecords.from_numpy(rec), getattr(Device, oname),
+                         [getattr(Device, dname)])
+        assert not out.status[0].cpu().numpy().any()
+        t = out.time_ns[0].cpu().numpy()
+        for i, r in enumerate(rows):
+            assert t[i] == pytest.approx(r["time_ns"], rel=TIME_RTOL), r
+            for key, col in (("occ_origin", out.occ_origin), ("occ_dest", out.occ_dest[0]),
+                             ("wave_origin", out.wave_origin), ("wave_dest", out.wave_dest[0])):
+                if key in r:
+                    assert int(col[i]) == r[key], (key, r)
+        # gamma alone for the rows that have metrics
+        from habitat_amd.analysis.wave_scaling.batch import roofline_gamma
+        g = roofline_gamma(KernelRecords.from_numpy(rec), getattr(Device, oname),
+                           getattr(Device, dname)).cpu().numpy()
+        for i, r in enumerate(rows):
+            if r.get("has_metrics", True):
+                assert g[i] == pytest.approx(r["gamma"], rel=1e-12), r
+
+
 def test_identity_and_round_trip_properties():
     rec, _ = synthetic.kernel_records(200_000, Device.V100, seed=3, metrics_fraction=0.5)
     kr = KernelRecords.from_numpy(rec)
