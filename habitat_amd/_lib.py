@@ -9,6 +9,8 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libhabitat_mi.so")
 
+ABI_VERSION = 101   # HBT_VERSION of include/habitat_mi.h this binding was written for
+
 HBT_OK, HBT_EINVAL, HBT_ESPEC, HBT_EHIP, HBT_ENOMEM, HBT_EALIGN, HBT_ESIZE = 0, -1, -2, -3, -4, -5, -6
 ST_OK, ST_ORIGIN_WAVE_ZERO, ST_DEST_WAVE_ZERO, ST_BAD_GAMMA, ST_ZERO_BLOCKS = 0, 1, 2, 3, 4
 
@@ -55,7 +57,7 @@ _SIGNATURES = {
     "hbt_wave_scale_sum": (C.c_int, [_P, C.c_int64] + [_P] * 12 + [C.c_int32, _P, _P, _P]),
     "hbt_roofline_gamma": (C.c_int, [C.POINTER(DeviceSpec), C.POINTER(DeviceSpec), C.c_int64,
                                      _P, _P, _P, _P, _P, _P]),
-    "hbt_ratio_scale": (C.c_int, [_P, C.c_int32, C.c_int32, _P, _P, _P, _P]),
+    "hbt_ratio_scale": (C.c_int, [_P, C.c_int32, C.c_int32, _P, C.c_int32, _P, _P, _P, _P, _P]),
     "hbt_mlp_create": (_P, [C.c_int32, C.c_int32, C.c_int32, C.POINTER(_P), C.POINTER(_P), _P, _P,
                             C.POINTER(C.c_int)]),
     "hbt_mlp_forward": (C.c_int, [_P, _P, C.c_int64, _P, _P]),
@@ -91,6 +93,11 @@ def lib():
         # to the runtime the kernels are launched on.
         import torch  # noqa: F401
         handle = C.CDLL(LIB_PATH)
+        handle.hbt_version.restype = C.c_int
+        if handle.hbt_version() != ABI_VERSION:
+            raise ImportError(
+                "habitat_amd: %s implements ABI %d, this package binds ABI %d - rebuild it with "
+                "`python -m habitat_amd.build`" % (LIB_PATH, handle.hbt_version(), ABI_VERSION))
         for name, (res, args) in list(_SIGNATURES.items()) + list(_OPTIONAL.items()):
             fn = getattr(handle, name)
             fn.restype = res

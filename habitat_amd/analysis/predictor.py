@@ -308,26 +308,31 @@ class Predictor:
                                     self._special_enqueue(kind, operations, dest_device))
 
     def _special_enqueue(self, kind, operations, dest_device):
-        """The MLP launch of _special_scale_many; returns its output, still on
-        the GPU: rows 2i and 2i+1 are operation i on the destination and on its
-        origin."""
+        """The MLP launch of _special_scale_many.  Operations with equal features
+        and origin share their two rows (destination, origin); returns (the
+        launch's output, still on the GPU, and each operation's row pair)."""
         pred = self._mlp(kind)
-        rows = []
+        rows, pair_of, pairs = [], {}, []
         dest_feats = get_device_features(dest_device.name, pred.device_params)
         for op in operations:
             a = _ARGUMENTS[kind](op)
             feats = [a[x] for x in pred.model.features]
-            rows.append(feats + dest_feats)
-            rows.append(feats + get_device_features(op.device.name, pred.device_params))
-        return pred.predict_batch(np.asarray(rows, np.float64))
+            key = (tuple(feats), op.device.name)
+            if key not in pair_of:
+                pair_of[key] = len(rows) // 2
+                rows.append(feats + dest_feats)
+                rows.append(feats + get_device_features(op.device.name, pred.device_params))
+            pairs.append(pair_of[key])
+        return pred.predict_batch(np.asarray(rows, np.float64)), pairs
 
     @staticmethod
-    def _special_finish(operations, y):
+    def _special_finish(operations, enqueued):
         """Measured time x predicted destination time / predicted origin time,
         not below zero (predictor.py:132-148)."""
+        y, pairs = enqueued
         y = y.cpu().numpy().astype(np.float64)
         out = []
-        for i, op in enumerate(operations):
+        for op, i in zip(operations, pairs):
             ms = op.run_time_ms * float(y[2 * i]) / float(y[2 * i + 1])
             if ms < 0:
                 logger.warning("Operation %s predicted run time %.2f ms", op.name, ms)

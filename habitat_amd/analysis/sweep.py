@@ -11,9 +11,12 @@ analysis/run_time.py:50-58, analysis/predictor.py:111-148)
 is computed once on the host.  The per-destination parts run on the GPU: one
 hbt_wave_scale_sum launch over all kernel records of the trace (scaled times
 are summed per pass on the fly and never written out), one MLP launch per
-operation kind over (destinations + origin) x operations rows, and
+operation kind over (destinations + origin) x distinct feature rows (a network
+repeats layer shapes: ResNet-50's 53 convolutions have 23 distinct rows), and
 hbt_ratio_scale for the ratio, clamp and sum.
 """
+import logging
+
 import numpy as np
 import torch
 
@@ -21,6 +24,8 @@ from habitat_amd.analysis import SPECIAL_OPERATIONS
 from habitat_amd.analysis.mlp.devices import get_device_features
 from habitat_amd.analysis.run_time import ms_to_ns
 from habitat_amd.analysis.wave_scaling.batch import DeviceTable, ratio_scale, wave_scale_sum
+
+logger = logging.getLogger(__name__)
 
 
 class TraceSweep:
@@ -35,6 +40,19 @@ class TraceSweep:
         self.special_ms = {}        # kind -> float64 [D, n_ops of that kind]
         self.special_owner = {}     # kind -> list of operation indices
         self.bad_records = None     # int32 [D]: records on which the reference would raise
+        self.clamped_ops = None     # int32 [D]: MLP operations predicted negative, counted as 0
+
+    def warn_if_clamped(self):
+        """The reference warns once per operation whose MLP prediction is
+        negative (predictor.py:135-141); a sweep counts them on the GPU and this
+        logs one line for the whole sweep.  Reads the counter back (synchronises).
+        Returns the counts as a list."""
+        counts = self.clamped_ops.cpu().tolist() if self.clamped_ops is not None else []
+        if any(counts):
+            logger.warning(
+                "%d MLP-predicted operation(s) had a negative predicted run time on %d of %d "
+                "devices and count as 0 ms", sum(counts), sum(1 for c in counts if c), len(counts))
+        return counts
 
 
 class TracePlan:
@@ -87,10 +105,13 @@ class TracePlan:
             for op in ops:
                 a = P._ARGUMENTS[kind](op)
                 feats.append([a[x] for x in pred.model.features])
+            # operations with equal features share one MLP row
+            uniq, op_row = np.unique(np.asarray(feats, np.float64), axis=0, return_inverse=True)
             self.special[kind] = (
                 idxs, pred,
-                torch.tensor(np.asarray(feats, np.float64), device=self.gpu),          # [O, F]
-                torch.tensor([op.run_time_ms for op in ops], dtype=torch.float64, device=self.gpu))
+                torch.tensor(uniq, device=self.gpu),                                   # [U, F]
+                torch.tensor([op.run_time_ms for op in ops], dtype=torch.float64, device=self.gpu),
+                torch.tensor(op_row.reshape(-1), dtype=torch.int32, device=self.gpu))  # [O]
 
     def _records_for(self, dest):
         """Kernel records with the register column resolved for `dest`'s
@@ -175,20 +196,23 @@ class SweepCall:
         # operations fills a fraction of the GPU, so the kinds run side by side.
         main = torch.cuda.current_stream(plan.gpu)
         preds = {}
-        for (kind, (idxs, pred, op_feats, ms)), side in zip(plan.special.items(), self.streams):
-            O = op_feats.shape[0]
+        for (kind, (idxs, pred, op_feats, ms, op_row)), side in zip(plan.special.items(),
+                                                                    self.streams):
+            U = op_feats.shape[0]
             side.wait_stream(main)
             with torch.cuda.stream(side):
-                rows = torch.cat([op_feats.unsqueeze(0).expand(D + 1, O, -1),
-                                  self.dev_feats.unsqueeze(1).expand(D + 1, O, 4)], dim=2)
-                y = pred.predict_batch(rows.reshape((D + 1) * O, -1)).view(D + 1, O)
+                rows = torch.cat([op_feats.unsqueeze(0).expand(D + 1, U, -1),
+                                  self.dev_feats.unsqueeze(1).expand(D + 1, U, 4)], dim=2)
+                y = pred.predict_batch(rows.reshape((D + 1) * U, -1)).view(D + 1, U)
             rows.record_stream(main)
             y.record_stream(main)
             preds[kind] = y
         for side in self.streams:
             main.wait_stream(side)
-        for kind, (idxs, pred, op_feats, ms) in plan.special.items():
-            res.special_ms[kind] = ratio_scale(preds[kind], ms, D, totals=total)
+        res.clamped_ops = torch.zeros((D,), dtype=torch.int32, device=plan.gpu)
+        for kind, (idxs, pred, op_feats, ms, op_row) in plan.special.items():
+            res.special_ms[kind] = ratio_scale(preds[kind], ms, D, totals=total, op_row=op_row,
+                                               clamped=res.clamped_ops)
             res.special_owner[kind] = idxs
         res.total_ms = total
         return res
@@ -203,4 +227,7 @@ def predict_trace_times(predictor, trace, dest_devices, device_features=None):
     optionally maps a device name to its four MLP features (default: the table
     of mlp/devices.py).  A destination on which the reference would raise yields
     NaN."""
-    return predict_trace_sweep(predictor, trace, dest_devices, device_features).total_ms.cpu().tolist()
+    sweep = predict_trace_sweep(predictor, trace, dest_devices, device_features)
+    totals = sweep.total_ms.cpu().tolist()
+    sweep.warn_if_clamped()
+    return totals

@@ -201,26 +201,37 @@ def wave_scale_sum(records, table, segment=None, n_segments=1, stream=None):
     return sums, bad
 
 
-def ratio_scale(pred, run_time_ms, n_dest, totals=None, want_ms=True, stream=None):
+def ratio_scale(pred, run_time_ms, n_dest, totals=None, want_ms=True, stream=None, op_row=None,
+                clamped=None):
     """MLP-predicted operations on a sweep (see hbt_ratio_scale).  pred: float32
-    GPU tensor [(n_dest + 1), n_ops] whose last row is the origin; run_time_ms:
-    float64 GPU tensor [n_ops].  Returns ms [n_dest, n_ops] (or None) and adds the
-    per-destination sums to `totals` ([n_dest] float64) if given."""
+    GPU tensor [(n_dest + 1), n_rows] whose last row is the origin; run_time_ms:
+    float64 GPU tensor [n_ops]; op_row: int32 GPU tensor [n_ops] naming each
+    operation's column of pred (None: column o, n_rows == n_ops).  Returns ms
+    [n_dest, n_ops] (or None), adds the per-destination sums to `totals`
+    ([n_dest] float64) and the number of negative predictions replaced by 0 to
+    `clamped` ([n_dest] int32) if given."""
     n_ops = run_time_ms.shape[0]
-    if pred.dtype != torch.float32 or tuple(pred.shape) != (n_dest + 1, n_ops):
+    n_rows = pred.shape[1] if pred.dim() == 2 else -1
+    if pred.dtype != torch.float32 or pred.dim() != 2 or pred.shape[0] != n_dest + 1 or (
+            op_row is None and n_rows != n_ops):
         raise TypeError("pred must be float32 [%d, %d]" % (n_dest + 1, n_ops))
+    if op_row is not None and (op_row.dtype != torch.int32 or op_row.shape != (n_ops,)):
+        raise TypeError("op_row must be int32 [%d]" % n_ops)
     if run_time_ms.dtype != torch.float64 or (totals is not None and (
             totals.dtype != torch.float64 or totals.shape != (n_dest,))):
         raise TypeError("run_time_ms and totals must be float64")
+    if clamped is not None and (clamped.dtype != torch.int32 or clamped.shape != (n_dest,)):
+        raise TypeError("clamped must be int32 [%d]" % n_dest)
     pred = pred.contiguous()
     out = (torch.empty((n_dest, n_ops), dtype=torch.float64, device=pred.device)
            if want_ms else None)
     if stream is None:
         stream = torch.cuda.current_stream(pred.device)
     with torch.cuda.device(pred.device):
-        rc = _lib.lib().hbt_ratio_scale(_ptr(pred), n_dest, n_ops, _ptr(run_time_ms.contiguous()),
-                                        _ptr(out), _ptr(totals),
-                                        ctypes.c_void_p(stream.cuda_stream))
+        rc = _lib.lib().hbt_ratio_scale(
+            _ptr(pred), n_dest, n_rows, _ptr(op_row.contiguous() if op_row is not None else None),
+            n_ops, _ptr(run_time_ms.contiguous()), _ptr(out), _ptr(totals), _ptr(clamped),
+            ctypes.c_void_p(stream.cuda_stream))
     _lib.check(rc, "hbt_ratio_scale")
     return out
 

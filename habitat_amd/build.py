@@ -25,6 +25,22 @@ HIPCC_FLAGS = [
 ]
 
 
+def sources():
+    """Every file the library is compiled from (sources and headers)."""
+    root = os.path.dirname(HERE)
+    files = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC))
+             if f.endswith((".hip", ".h"))]
+    return files + [os.path.join(root, "include", "habitat_mi.h")]
+
+
+def is_stale():
+    """True when there is no library or a source file is newer than it."""
+    if not os.path.exists(LIB_PATH):
+        return True
+    built = os.path.getmtime(LIB_PATH)
+    return any(os.path.getmtime(f) > built for f in sources() if os.path.exists(f))
+
+
 def build(verbose=False):
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     os.makedirs(LIB_DIR, exist_ok=True)

@@ -80,7 +80,13 @@ int hbt_device_spec_check(const hbt_device_spec* s) {
   if (s->smem_per_sm < 0 || s->smem_per_sm >= two31) return HBT_ESPEC;
   if (s->smem_per_block_optin < 0 || s->smem_per_block_optin >= two31) return HBT_ESPEC;
   if (s->warp_size > 32768) return HBT_ESPEC;
-  if (s->num_sms > (1 << 26)) return HBT_ESPEC;
+  // wave size = num_sms x occupancy (at most 63) is formed in 24-bit arithmetic
+  if (s->num_sms > (1 << 20)) return HBT_ESPEC;
+  // An AMD compute-unit description holds as many one-wave work-groups as it
+  // has wave slots; the small-kernel factor's logarithm table ends at 63.
+  if (s->compute_major == HBT_COMPUTE_MAJOR_CDNA && s->warp_size > 0 &&
+      s->max_threads_per_sm / s->warp_size > 63)
+    return HBT_ESPEC;
   const double f[3] = {s->mem_bandwidth_gb, s->base_clock_mhz, s->peak_gflops};
   for (double v : f)
     if (!(v > 0) || !std::isfinite(v)) return HBT_ESPEC;

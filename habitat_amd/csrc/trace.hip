@@ -13,8 +13,8 @@
 //                        in L2) plus 8 bytes per (destination, segment).
 //   hbt_ratio_scale      per destination and MLP-predicted operation:
 //                        run_time_ms * pred_dest / pred_origin, negative -> 0
-//                        (predictor.py:132-148 and :182,218,238,283), and the
-//                        per-destination sum of those.
+//                        (predictor.py:132-148 and :182,218,238,283), the
+//                        per-destination sum of those and the number replaced.
 //
 // Destinations live in a device-resident table (hbt_device_table) so that one
 // launch covers all of them: blockIdx.y is the destination, and its constants
@@ -161,36 +161,59 @@ __global__ __launch_bounds__(kBlock) void roofline_gamma_kernel(const GammaArgs 
 }
 
 struct RatioArgs {
-  const float* pred;          // [(n_dest + 1)][n_ops]; the last row is the origin
+  const float* pred;          // [(n_dest + 1)][n_rows]; the last row is the origin
   const double* run_time_ms;  // [n_ops]
-  int32_t n_dest, n_ops;
+  const int32_t* op_row;      // [n_ops], nullable: operation o reads column o
+  int32_t n_dest, n_rows, n_ops;
   double* out_ms;             // [n_dest][n_ops], nullable
   double* out_total;          // [n_dest], nullable; added to
+  int32_t* out_clamped;       // [n_dest], nullable; added to
 };
 
 // blockIdx.x = destination; the block's threads stride over the operations.
+// Operations with equal features share one column of pred.
 __global__ __launch_bounds__(kBlock) void ratio_scale_kernel(const RatioArgs a) {
   const int d = blockIdx.x;
-  const float* dest = a.pred + (int64_t)d * a.n_ops;
-  const float* orig = a.pred + (int64_t)a.n_dest * a.n_ops;
+  const float* dest = a.pred + (int64_t)d * a.n_rows;
+  const float* orig = a.pred + (int64_t)a.n_dest * a.n_rows;
   double acc = 0.0;
+  int32_t clamped = 0;
   for (int o = threadIdx.x; o < a.n_ops; o += kBlock) {
-    // predictor.py:182: operation.run_time_ms * pred_dest / pred_orig, in fp64
-    double ms = a.run_time_ms[o] * (double)dest[o] / (double)orig[o];
-    ms = (ms < 0) ? 0. : ms;   // predictor.py:135-141
+    const int32_t row = a.op_row != nullptr ? a.op_row[o] : o;
+    double ms = __builtin_nan("");
+    if (row >= 0 && row < a.n_rows) {
+      // predictor.py:182: operation.run_time_ms * pred_dest / pred_orig, in fp64
+      ms = a.run_time_ms[o] * (double)dest[row] / (double)orig[row];
+      if (ms < 0) {   // predictor.py:135-141: warned about and replaced by 0
+        ms = 0.;
+        ++clamped;
+      }
+    }
     if (a.out_ms != nullptr) a.out_ms[(int64_t)d * a.n_ops + o] = ms;
     acc += ms;
   }
-  if (a.out_total == nullptr) return;
+  if (a.out_total == nullptr && a.out_clamped == nullptr) return;
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off);
+  for (int off = 32; off > 0; off >>= 1) {
+    acc += __shfl_down(acc, off);
+    clamped += __shfl_down(clamped, off);
+  }
   __shared__ double part[kBlock / 64];
-  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+  __shared__ int32_t part_clamped[kBlock / 64];
+  if ((threadIdx.x & 63) == 0) {
+    part[threadIdx.x >> 6] = acc;
+    part_clamped[threadIdx.x >> 6] = clamped;
+  }
   __syncthreads();
   if (threadIdx.x == 0) {
     double total = 0.0;
-    for (int w = 0; w < kBlock / 64; ++w) total += part[w];
-    a.out_total[d] += total;
+    int32_t count = 0;
+    for (int w = 0; w < kBlock / 64; ++w) {
+      total += part[w];
+      count += part_clamped[w];
+    }
+    if (a.out_total != nullptr) a.out_total[d] += total;
+    if (a.out_clamped != nullptr) a.out_clamped[d] += count;
   }
 }
 
@@ -345,14 +368,18 @@ int hbt_roofline_gamma(const hbt_device_spec* origin, const hbt_device_spec* des
   return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
 }
 
-int hbt_ratio_scale(const float* pred, int32_t n_dest, int32_t n_ops, const double* run_time_ms,
-                    double* out_ms, double* out_total, void* hip_stream) {
+int hbt_ratio_scale(const float* pred, int32_t n_dest, int32_t n_rows, const int32_t* op_row,
+                    int32_t n_ops, const double* run_time_ms, double* out_ms, double* out_total,
+                    int32_t* out_clamped, void* hip_stream) {
   using namespace hbt;
-  if (n_dest < 0 || n_ops < 0) return HBT_EINVAL;
+  if (n_dest < 0 || n_ops < 0 || n_rows < 0) return HBT_EINVAL;
+  if (op_row == nullptr && n_rows != n_ops) return HBT_EINVAL;
   if (n_dest == 0 || n_ops == 0) return HBT_OK;
-  if (pred == nullptr || run_time_ms == nullptr || (out_ms == nullptr && out_total == nullptr))
+  if (pred == nullptr || run_time_ms == nullptr ||
+      (out_ms == nullptr && out_total == nullptr && out_clamped == nullptr))
     return HBT_EINVAL;
-  RatioArgs a{pred, run_time_ms, n_dest, n_ops, out_ms, out_total};
+  if (n_rows == 0) return HBT_EINVAL;
+  RatioArgs a{pred, run_time_ms, op_row, n_dest, n_rows, n_ops, out_ms, out_total, out_clamped};
   hipLaunchKernelGGL(ratio_scale_kernel, dim3((unsigned)n_dest), dim3(kBlock), 0,
                      static_cast<hipStream_t>(hip_stream), a);
   return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;

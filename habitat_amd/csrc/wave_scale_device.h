@@ -21,12 +21,15 @@
 namespace hbt {
 namespace dev {
 
-// log2(i) for i = 0..32 (entry 0 unused), padded to one entry per lane.  A
-// kernel that fits in one wave on a device has num_blocks < num_sms * occupancy
-// with occupancy <= 32 block slots, so ceil(num_blocks / num_sms) is an integer
-// in 1..32 and the logarithm of the small-kernel factor needs no more than this
-// table.  Each wavefront keeps it in one register pair (lane i holds entry i)
-// and looks entries up with a cross-lane permute: no LDS, no barrier.
+// log2(i) for i = 0..63 (entry 0 unused), one entry per lane.  A kernel that
+// fits in one wave on a device has num_blocks < num_sms * occupancy, so
+// ceil(num_blocks / num_sms) is an integer in 1..occupancy.  NVIDIA-rule
+// devices hold at most 32 blocks per SM; an AMD compute-unit description holds
+// as many one-wave work-groups as it has wave slots, and hbt_device_spec_check
+// keeps those at 63 or fewer (40 on a CU with 10 waves per SIMD), so the
+// logarithm of the small-kernel factor needs no more than this table.  Each
+// wavefront keeps it in one register pair (lane i holds entry i) and looks
+// entries up with a cross-lane permute: no LDS, no barrier.
 __device__ static const double kLog2Int[64] = {
     0x0.0p+0, 0x0.0p+0, 0x1.0000000000000p+0, 0x1.95c01a39fbd68p+0, 0x1.0000000000000p+1,
     0x1.2934f0979a371p+1, 0x1.4ae00d1cfdeb4p+1, 0x1.675767f54042dp+1, 0x1.8000000000000p+1,
@@ -35,7 +38,15 @@ __device__ static const double kLog2Int[64] = {
     0x1.0598fdbeb244cp+2, 0x1.0ae00d1cfdeb4p+2, 0x1.0fde0b5c81340p+2, 0x1.149a784bcd1b9p+2,
     0x1.191bba891f171p+2, 0x1.1d6753e032ea1p+2, 0x1.21820a01ac755p+2, 0x1.2570068e7ef5ap+2,
     0x1.2934f0979a371p+2, 0x1.2cd4011c8f119p+2, 0x1.305013ab7ce0ep+2, 0x1.33abb3faa0216p+2,
-    0x1.36e9291eaa65bp+2, 0x1.3a0a7eda4c113p+2, 0x1.3d118d66c4d4ep+2, 0x1.4000000000000p+2};
+    0x1.36e9291eaa65bp+2, 0x1.3a0a7eda4c113p+2, 0x1.3d118d66c4d4ep+2, 0x1.4000000000000p+2,
+    0x1.42d75a6eb1dfbp+2, 0x1.4598fdbeb244cp+2, 0x1.48462c466d3cfp+2, 0x1.4ae00d1cfdeb4p+2,
+    0x1.4d67af16da765p+2, 0x1.4fde0b5c81340p+2, 0x1.524407ab0e074p+2, 0x1.549a784bcd1b9p+2,
+    0x1.56e221cd9d0cep+2, 0x1.591bba891f171p+2, 0x1.5b47ebf73882ap+2, 0x1.5d6753e032ea1p+2,
+    0x1.5f7a8568cb06dp+2, 0x1.61820a01ac755p+2, 0x1.637e623d2ba02p+2, 0x1.6570068e7ef5ap+2,
+    0x1.675767f54042dp+2, 0x1.6934f0979a371p+2, 0x1.6b09044d313a6p+2, 0x1.6cd4011c8f119p+2,
+    0x1.6e963fac9c0eap+2, 0x1.705013ab7ce0ep+2, 0x1.7201cc2c0005ap+2, 0x1.73abb3faa0216p+2,
+    0x1.754e11eb0029ap+2, 0x1.76e9291eaa65bp+2, 0x1.787d3945c340bp+2, 0x1.7a0a7eda4c113p+2,
+    0x1.7b9133567feaep+2, 0x1.7d118d66c4d4ep+2, 0x1.7e8bc1179e0cbp+2};
 
 struct RecordIn {
   int32_t nb, block, smem_total, regs, dest_regs;
@@ -234,7 +245,7 @@ struct RecordOut {
 
 // Written with selects rather than branches: the 64 records of a wavefront
 // take all paths between them anyway.
-// log2 of a small-kernel block count (0..32).  PERMUTE: read it from the lane
+// log2 of a small-kernel block count (0..63).  PERMUTE: read it from the lane
 // that holds it (needs all 64 lanes of the wavefront active); otherwise gather
 // it from the table in memory.
 template <bool PERMUTE>
@@ -292,7 +303,7 @@ __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn
   o.status = (uint8_t)status;
 
   // roofline.py:32-45: (clk_ratio * dest_max_occ / origin_max_occ)^(1-gamma), both
-  // counts in 1..32; roofline.py:48-64: bw^gamma * clk^(1-gamma) * sm^(1-gamma)
+  // counts in 1..63; roofline.py:48-64: bw^gamma * clk^(1-gamma) * sm^(1-gamma)
   const double gamma_compl = 1.0 - gamma;
   const double log2_small = p.log2_clk + log2_count<PERMUTE>(log2_lane, dest_max_occ) -
                             log2_count<PERMUTE>(log2_lane, m.origin_max_occ);

@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define HBT_VERSION 100 /* 0.1.0 */
+#define HBT_VERSION 101 /* 0.1.1 */
 
 enum {
   HBT_OK = 0,
@@ -88,8 +88,11 @@ int hbt_device_count(void);
 
 /*
  * HBT_OK when `spec` (host) is inside the domain the batch kernels accept:
- * smem fields >= 0 and < 2^31, warp_size <= 32768, num_sms <= 2^26,
- * mem_bandwidth_gb, base_clock_mhz, peak_gflops finite and > 0.  A spec the
+ * smem fields >= 0 and < 2^31, warp_size <= 32768, num_sms <= 2^20,
+ * mem_bandwidth_gb, base_clock_mhz, peak_gflops finite and > 0, and for an AMD
+ * compute-unit description (HBT_COMPUTE_MAJOR_CDNA) at most 63 wave slots per
+ * CU (max_threads_per_sm / warp_size; 32 on gfx90a and later, 40 on CUs with 10
+ * waves per SIMD).  A spec the
  * occupancy model rejects (unknown compute capability, a zero limit) is still
  * in the domain: every occupancy on it is 0, as in the reference.
  */
@@ -209,13 +212,19 @@ int hbt_roofline_gamma(const hbt_device_spec *origin, const hbt_device_spec *des
 /*
  * The last step of the MLP-predicted operations for a device sweep
  * (analysis/predictor.py:132-148 with :182,218,238,283): pred is
- * [(n_dest + 1)][n_ops] fp32 MLP outputs, the last row evaluated with the
- * origin's device features; out_ms[d][o] = run_time_ms[o] * pred[d][o] /
- * pred[n_dest][o] in fp64, negative values replaced by 0 (out_ms nullable), and
- * out_total[d] += sum over o of out_ms[d][o] (nullable).
+ * [(n_dest + 1)][n_rows] fp32 MLP outputs, the last row evaluated with the
+ * origin's device features; operation o reads column op_row[o] (device,
+ * [n_ops], nullable = column o, then n_rows must equal n_ops), so operations
+ * with equal features share one MLP row.  out_ms[d][o] = run_time_ms[o] *
+ * pred[d][r] / pred[n_dest][r] in fp64, negative values replaced by 0 (out_ms
+ * nullable); out_total[d] += sum over o of out_ms[d][o] (nullable);
+ * out_clamped[d] += the number of operations whose value was negative
+ * (nullable): the reference logs a warning for each of them
+ * (predictor.py:135-141).  A column index outside [0, n_rows) gives NaN.
  */
-int hbt_ratio_scale(const float *pred, int32_t n_dest, int32_t n_ops, const double *run_time_ms,
-                    double *out_ms, double *out_total, void *hip_stream);
+int hbt_ratio_scale(const float *pred, int32_t n_dest, int32_t n_rows, const int32_t *op_row,
+                    int32_t n_ops, const double *run_time_ms, double *out_ms, double *out_total,
+                    int32_t *out_clamped, void *hip_stream);
 
 /*
  * Per-operation MLP (fc1 -> ReLU -> hidden x (Linear, ReLU) -> fc2), the

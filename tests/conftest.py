@@ -18,10 +18,14 @@ def pytest_configure(config):
 
 @pytest.fixture(scope="session", autouse=True)
 def built_library():
-    """The tests load the library that is built; they compile it (hipcc
-    cross-compiles without a GPU) only when there is none."""
+    """The tests load the library that is built.  They compile it (hipcc
+    cross-compiles without a GPU) when there is none; on a machine without a
+    GPU, where sources get edited, also when a source file is newer than the
+    library, so that a stale build is not what gets tested.  A GPU box runs
+    the library it was sent."""
+    import torch
     from habitat_amd import _lib, build
-    if not os.path.exists(_lib.LIB_PATH):
+    if not os.path.exists(_lib.LIB_PATH) or (torch.cuda.device_count() == 0 and build.is_stale()):
         build.build()
     return _lib.LIB_PATH
 

@@ -184,6 +184,91 @@ def test_predictor_on_resnet50_shaped_trace():
         predicted.operations[0].to_device(origin, predictor)
 
 
+def test_bmm_lstm_and_every_call_form_against_hand_listed_features():
+    """A trace holding every case of tests/arguments_kat.py (conv2d with tuple,
+    int and keyword arguments, linear with 2 to 4 input dimensions, bmm, lstm
+    unpacked and packed) through Trace.to_device, Trace.to_devices and the
+    reference's per-operation private scalers.  The expected value feeds the
+    oracle the feature lists written by hand there and the device rows of
+    analysis/mlp/devices.csv:6-7 typed here, not the package's extraction."""
+    from arguments_kat import CASES, arguments_of
+    from habitat_amd.analysis.operation import MeasuredOperation
+    from habitat_amd.analysis.run_time import RunTimeMeasurement
+    device_rows = {"V100": [16, 900, 80, 14.028], "T4": [16, 320, 40, 8.1],
+                   "P100": [16, 732, 56, 9.3]}
+    origin = Device.V100
+    preds = seeded_predictors()
+    predictor = Predictor(mlp_predictors=preds)
+    ops = [MeasuredOperation(case[0], arguments_of(case),
+                             RunTimeMeasurement(0.5 + 0.25 * i, [], origin), None, origin)
+           for i, case in enumerate(CASES)]
+    trace = Trace(origin, ops)
+
+    def want_ms(i, dest):
+        kind, feats = CASES[i][0], CASES[i][5]
+        rp = preds[kind]
+        rows = np.array([feats + device_rows[dest.name], feats + device_rows["V100"]], np.float64)
+        y = omlp.forward_fp64(rp.model.state_dict(), rows, rp.mu, rp.sigma)
+        return opred.special_op_ms(ops[i].run_time_ms, y[0], y[1]), tolerance_ms(i, y)
+
+    def tolerance_ms(i, y):
+        # each fp32 network output is within 1e-4 of max(|y|, 1e-3) (the MLP
+        # tests' bar); the quotient of two of them carries both errors
+        err = [1e-4 * max(abs(v), 1e-3) / abs(v) for v in y]
+        return abs(ops[i].run_time_ms * y[0] / y[1]) * (err[0] + err[1]) * 1.01
+
+    for dest in (Device.T4, Device.P100):
+        predicted = trace.to_device(dest, predictor)
+        want = [want_ms(i, dest) for i in range(len(CASES))]
+        for case, op, (w, tol) in zip(CASES, predicted.operations, want):
+            assert op.backward is None and op.device is dest
+            assert abs(op.run_time_ms - w) <= tol, case[:2]
+        assert abs(predicted.run_time_ms - opred.trace_ms([w for w, _ in want])) <= sum(
+            t for _, t in want)
+    # the device sweep extracts its rows through the same functions
+    totals = trace.to_devices([Device.T4, Device.P100], predictor)
+    for dest, total in zip((Device.T4, Device.P100), totals):
+        want = [want_ms(i, dest) for i in range(len(CASES))]
+        assert abs(total - opred.trace_ms([w for w, _ in want])) <= sum(t for _, t in want)
+    # Exact networks make every feature position count: fc1 copies input j to
+    # unit j, the hidden layers are identities, fc2 weighs operation feature j
+    # with j + 2 and the SM count with 1000 (no normalisation), so a prediction
+    # is the integer  sum (j + 2) f_j + 1000 num_sms  and a wrong, swapped or
+    # shifted feature changes the quotient far beyond fp64 rounding.
+    exact = {}
+    for kind, rp in seeded_predictors().items():
+        n_op = len(rp.model.features)
+        with torch.no_grad():
+            for prm in rp.model.parameters():
+                prm.zero_()
+            for j in range(n_op + 4):
+                rp.model.fc1.weight[j, j] = 1.0
+            for layer in list(rp.model.mlp.layers)[::2]:
+                layer.weight.copy_(torch.eye(1024))
+            for j in range(n_op):
+                rp.model.fc2.weight[0, j] = float(j + 2)
+            rp.model.fc2.weight[0, n_op + 2] = 1000.0
+        rp.set_normalization(np.zeros(n_op + 4), np.ones(n_op + 4))
+        exact[kind] = rp
+    exact_predictor = Predictor(mlp_predictors=exact)
+    sms = {"V100": 80, "T4": 40, "P100": 56}
+    for dest in (Device.T4, Device.P100):
+        predicted = trace.to_device(dest, exact_predictor)
+        swept = exact_predictor.predict_trace_sweep(trace, [dest])
+        for i, (case, op) in enumerate(zip(CASES, predicted.operations)):
+            a = sum((j + 2) * f for j, f in enumerate(case[5]))
+            want = ops[i].run_time_ms * (a + 1000 * sms[dest.name]) / (a + 1000 * sms["V100"])
+            assert op.run_time_ms == pytest.approx(want, rel=1e-12), case[:2]
+        assert float(swept.total_ms[0]) == pytest.approx(predicted.run_time_ms, rel=1e-12)
+    # the reference's private per-operation scalers (predictor.py:150-283)
+    scalers = {"conv2d": predictor._conv2d_scale, "linear": predictor._linear_scale,
+               "bmm": predictor._bmm_scale, "lstm": predictor._lstm_scale}
+    for i, case in enumerate(CASES):
+        got = predictor._special_scale(ops[i], Device.T4, scalers[case[0]])
+        w, tol = want_ms(i, Device.T4)
+        assert abs(got.run_time_ms - w) <= tol, case[:2]
+
+
 def test_predictor_with_a_caller_supplied_strategy_and_pass_through_ops():
     from habitat_amd.analysis.arguments import Arguments
     from habitat_amd.analysis.operation import MeasuredOperation

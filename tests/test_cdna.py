@@ -97,6 +97,8 @@ def test_host_and_32_bit_model_follow_the_restatement():
     variants.append(dict(variants[0], compute_minor=4, shared_mem_per_block=65536,
                          shared_mem_per_multiprocessor=65536, num_sms=304))      # MI300X-like
     variants.append(dict(variants[0], compute_minor=0, warp_size=48))            # non power of two
+    variants.append(dict(variants[0], compute_minor=0, max_threads_per_multiprocessor=2560,
+                         num_sms=120))                                # 10 waves per SIMD: 40 slots
     variants.append(dict(variants[0], regs_per_multiprocessor=0))                # rejected
     for props in variants:
         dev = DeviceProperties(name="v", **props)
@@ -156,6 +158,67 @@ def test_kernel_scales_with_compute_unit_occupancies(origin_name, dest_name):
             assert t[i] == pytest.approx(want, rel=1e-6)
             n_ok += 1
     assert n_ok > 1000
+
+
+@pytest.mark.gpu
+def test_small_kernels_on_a_compute_unit_with_forty_wave_slots():
+    """A CU with 10 waves per SIMD holds 40 one-wave work-groups, so a kernel
+    that fits one wave there can have ceil(num_blocks / CUs) anywhere in 1..40:
+    the small-kernel factor's logarithms beyond 32 (NVIDIA's block-slot limit)
+    are exercised on the origin and on the destination side, through the
+    straight-line instantiations, the general one and the fused sums."""
+    import torch
+    from habitat_amd.analysis.wave_scaling.batch import (DeviceTable, KernelRecords, wave_scale,
+                                                         wave_scale_sum)
+    from oracle import wave_scaling as ows
+    forty = DeviceProperties(name="forty", **dict(
+        Device.MI355X_cdna.as_dict(), compute_minor=0, max_threads_per_multiprocessor=2560,
+        num_sms=120, mem_bandwidth_gb=1200, base_clock_mhz=1500, peak_gflops_per_second=23000))
+    assert forty.thread_block_occupancy(64, 0, 0, 32) == 40
+    rng = np.random.default_rng(8)
+    n = 6000
+    rec = {"num_blocks": rng.integers(1, 41 * 120, n).astype(np.int32),
+           "block_size": rng.choice([32, 64, 64, 64, 128], n).astype(np.int32),
+           "dynamic_smem": np.zeros(n, np.int32), "static_smem": np.zeros(n, np.int32),
+           "regs_per_thread": rng.integers(8, 56, n).astype(np.int32),
+           "run_time_ns": np.floor(10.0 ** rng.uniform(3, 7, n)),
+           "flop_sp_efficiency": 10.0 ** rng.uniform(-2, 2, n),
+           "dram_read_bytes": np.floor(10.0 ** rng.uniform(3, 10, n)),
+           "dram_write_bytes": np.floor(10.0 ** rng.uniform(3, 10, n)),
+           "has_metrics": (rng.random(n) < 0.8).astype(np.uint8)}
+    big = DeviceProperties(name="bigger", **dict(forty.as_dict(), num_sms=150))
+    kr = KernelRecords.from_numpy(rec)
+    for origin, dests in ((forty, [big]), (big, [forty]), (forty, [Device.MI355X_cdna]),
+                          (Device.V100, [forty]), (forty, [big, Device.V100])):
+        out = wave_scale(kr, origin, dests)
+        o = oracle_device(origin.as_dict())
+        ds = [oracle_device(d.as_dict()) for d in dests]
+        props = {id(o): origin.as_dict()}
+        props.update({id(d): dev.as_dict() for d, dev in zip(ds, dests)})
+        occupancy = _oracle_occupancy(props)
+        sums, bad = wave_scale_sum(kr, DeviceTable(origin, dests))
+        for di, d in enumerate(ds):
+            t = out.time_ns[di].cpu().numpy()
+            st = out.status[di].cpu().numpy()
+            beyond = total = 0
+            for i in range(n):
+                row = {k: v[i].item() for k, v in rec.items()}
+                want, status = ows.unified_with_status(
+                    row, o, d, has_metrics=bool(rec["has_metrics"][i]), occupancy=occupancy)
+                assert st[i] == status
+                if status == 0:
+                    assert t[i] == pytest.approx(want, rel=1e-6), row
+                    total += want
+                    wave_o = origin.num_sms * occupancy(o, row, row["regs_per_thread"])
+                    wave_d = dests[di].num_sms * occupancy(d, row, row["regs_per_thread"])
+                    nb = row["num_blocks"]
+                    if nb < wave_o and nb < wave_d and max(-(-nb // origin.num_sms),
+                                                           -(-nb // dests[di].num_sms)) > 32:
+                        beyond += 1
+            if origin is not Device.V100 and dests[di] is not Device.V100:
+                assert beyond > 50, (origin.name, dests[di].name)
+            assert sums[di, 0].item() == pytest.approx(total, rel=1e-9)
+            assert int(bad[di].item()) == int((st != 0).sum())
 
 
 @pytest.mark.gpu

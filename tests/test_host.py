@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     handle = ctypes.CDLL(_lib.LIB_PATH)
     for name in declared:
         assert hasattr(handle, name), name
-    assert _lib.lib().hbt_version() == 100
+    assert _lib.lib().hbt_version() == _lib.ABI_VERSION
     assert _lib.strerror(0) == "ok" and "spec" in _lib.strerror(_lib.HBT_ESPEC)
 
 
@@ -114,10 +114,19 @@ def test_spec_check_and_argument_errors():
     assert L.hbt_device_spec_check(None) == _lib.HBT_EINVAL
     for field, value in (("mem_bandwidth_gb", 0.0), ("base_clock_mhz", float("nan")),
                          ("peak_gflops", -1.0), ("warp_size", 1 << 16), ("smem_per_sm", -1),
-                         ("num_sms", 1 << 27)):
+                         ("num_sms", 1 << 27), ("num_sms", (1 << 20) + 1)):
         s = _lib.DeviceSpec.from_buffer_copy(ok)
         setattr(s, field, value)
         assert L.hbt_device_spec_check(ctypes.byref(s)) == _lib.HBT_ESPEC, field
+    s = _lib.DeviceSpec.from_buffer_copy(ok)
+    s.num_sms = 1 << 20
+    assert L.hbt_device_spec_check(ctypes.byref(s)) == 0
+    # an AMD compute-unit description may have up to 63 wave slots per CU
+    amd = Device.MI355X_cdna.spec
+    for slots, want in ((32, 0), (40, 0), (63, 0), (64, _lib.HBT_ESPEC)):
+        s = _lib.DeviceSpec.from_buffer_copy(amd)
+        s.max_threads_per_sm = slots * s.warp_size
+        assert L.hbt_device_spec_check(ctypes.byref(s)) == want, slots
     # a device the occupancy model rejects is still a valid spec: occupancy 0
     s = _lib.DeviceSpec.from_buffer_copy(ok)
     s.compute_major = 8
@@ -330,3 +339,30 @@ def test_prediction_from_times_matches_one_from_kernels():
     assert [k.name for k in lazy.kernels] == ["k0", "k1", "k2"]
     assert lazy.kernels is lazy.kernels and lazy.ktime_ns == eager.ktime_ns
     assert lazy.device is dev
+
+
+def test_feature_extraction_known_answers():
+    """Recorded call shapes -> MLP feature rows, against lists written by hand
+    from the reference's four scalers (tests/arguments_kat.py): conv2d with
+    tuple / int / keyword arguments, linear with 2, 3 and 4 input dimensions,
+    bmm, both lstm overloads."""
+    from arguments_kat import CASES, FEATURE_ORDER, arguments_of
+    from habitat_amd.analysis import predictor as P
+    from habitat_amd.analysis.mlp import mlp as M
+    from habitat_amd.analysis.operation import MeasuredOperation
+    from habitat_amd.analysis.run_time import RunTimeMeasurement
+    classes = {"conv2d": M.Conv2DMLP, "linear": M.LinearMLP, "bmm": M.BMMMLP, "lstm": M.LSTMMLP}
+    for kind, cls in classes.items():
+        assert list(cls(1, 8).features) == FEATURE_ORDER[kind]
+    seen = set()
+    for case in CASES:
+        kind, label, _, _, _, want = case
+        op = MeasuredOperation(kind, arguments_of(case),
+                               RunTimeMeasurement(1.0, [], Device.V100), None, Device.V100)
+        named = P._ARGUMENTS[kind](op)
+        assert sorted(named) == sorted(FEATURE_ORDER[kind]), label
+        got = [named[x] for x in FEATURE_ORDER[kind]]
+        assert got == want, (kind, label, got)
+        assert all(type(v) is int for v in got), (kind, label)
+        seen.add(kind)
+    assert seen == set(classes)

@@ -91,6 +91,93 @@ def test_ratio_scale_matches_python_arithmetic():
         assert np.array_equal(out[d], np.array(want))            # same fp64 operations
         assert totals[d].item() == pytest.approx(2.5 + sum(want), rel=1e-12)
     assert (out == 0).any()
+    # operations that share MLP rows: column op_row[o] of pred; the negative
+    # predictions the reference warns about (predictor.py:135-141) are counted
+    U = 40
+    op_row = rng.integers(0, U, O).astype(np.int32)
+    shared = np.ascontiguousarray(pred[:, :U])
+    totals = torch.zeros((D,), dtype=torch.float64, device="cuda")
+    clamped = torch.full((D,), 3, dtype=torch.int32, device="cuda")
+    out = ratio_scale(torch.from_numpy(shared).cuda(), torch.from_numpy(ms).cuda(), D,
+                      totals=totals, op_row=torch.from_numpy(op_row).cuda(),
+                      clamped=clamped).cpu().numpy()
+    for d in range(D):
+        raw = [ms[o] * float(shared[d, op_row[o]]) / float(shared[D, op_row[o]]) for o in range(O)]
+        want = [opred.special_op_ms(ms[o], float(shared[d, op_row[o]]), float(shared[D, op_row[o]]))
+                for o in range(O)]
+        assert np.array_equal(out[d], np.array(want))
+        assert totals[d].item() == pytest.approx(sum(want), rel=1e-12)
+        assert clamped[d].item() == 3 + sum(1 for v in raw if v < 0)
+    assert int(clamped.sum().item()) > 3 * D
+    # a column index outside the table gives NaN instead of a stray read
+    op_row[5] = U
+    op_row[6] = -1
+    out = ratio_scale(torch.from_numpy(shared).cuda(), torch.from_numpy(ms).cuda(), D,
+                      op_row=torch.from_numpy(op_row).cuda()).cpu().numpy()
+    assert np.isnan(out[:, 5]).all() and np.isnan(out[:, 6]).all()
+    assert not np.isnan(np.delete(out, [5, 6], axis=1)).any()
+    # counters alone
+    only = torch.zeros((D,), dtype=torch.int32, device="cuda")
+    assert ratio_scale(torch.from_numpy(pred).cuda(), torch.from_numpy(ms).cuda(), D,
+                       want_ms=False, clamped=only) is None
+    assert only.cpu().tolist() == [int((pred[d] < 0).sum()) for d in range(D)]
+
+
+def test_sweep_shares_rows_of_equal_operations_and_counts_clamped_ones(caplog):
+    """ResNet-50 repeats its layer shapes: the sweep evaluates each distinct
+    feature row once per device and every operation still gets its own time.
+    A network that predicts negative times on some devices is clamped to 0 and
+    counted, with one warning for the sweep (the reference warns per operation,
+    predictor.py:135-141)."""
+    import logging
+    predictor, trace, devices, feats = _sweep_fixture(12)
+    plan = predictor.plan_trace(trace)
+    idxs, pred, op_feats, ms, op_row = plan.special["conv2d"]
+    assert len(idxs) == 53 and op_feats.shape[0] < 53          # shared rows
+    assert op_row.shape == (53,) and int(op_row.max()) == op_feats.shape[0] - 1
+    sweep = plan.run(devices, feats)
+    per_op = sweep.special_ms["conv2d"].cpu().numpy()
+    assert per_op.shape == (12, 53)
+    assert int(sweep.clamped_ops.sum().item()) == 0
+    # against one operation at a time on three of the devices
+    from habitat_amd.analysis.mlp import devices as md
+    try:
+        for d, f in zip(devices, synthetic.device_sweep(12, seed=1)[1]):
+            md.register_device(d.name, *f)
+        for di in (0, 5, 11):
+            for col in (0, 17, 52):
+                op = trace.operations[idxs[col]]
+                single = predictor.predict_operation(op, devices[di]).run_time_ms
+                assert per_op[di, col] == pytest.approx(single, rel=1e-5)
+    finally:
+        for d in devices:
+            md.unregister_device(d.name)
+    # a network whose output is  num_sms - 100  (no normalisation): negative on
+    # every device with fewer than 100 SMs, positive on the origin's copy of 150
+    rp = predictor.conv2d_pred
+    with torch.no_grad():
+        for prm in rp.model.parameters():
+            prm.zero_()
+        rp.model.fc1.weight[0, 10] = 1.0
+        for layer in list(rp.model.mlp.layers)[::2]:
+            layer.weight.copy_(torch.eye(1024))
+        rp.model.fc2.weight[0, 0] = 1.0
+        rp.model.fc2.bias.fill_(-100.0)
+    rp.set_normalization(np.zeros(12), np.ones(12))
+    feats = dict(feats)
+    feats[Device.V100.name] = [16, 900, 150, 14.028]
+    with caplog.at_level(logging.WARNING, logger="habitat_amd.analysis.sweep"):
+        totals = predictor.predict_trace_times(trace, devices, feats)
+    sweep = predictor.predict_trace_sweep(trace, devices, feats)
+    counts = sweep.clamped_ops.cpu().tolist()
+    small = [f[2] < 100 for f in synthetic.device_sweep(12, seed=1)[1]]
+    assert any(small) and not all(small)
+    assert counts == [53 if s else 0 for s in small]
+    per_op = sweep.special_ms["conv2d"].cpu().numpy()
+    for di, s in enumerate(small):
+        assert (per_op[di] == 0).all() == s
+    assert sum("negative predicted run time" in r.message for r in caplog.records) == 1
+    assert np.isfinite(totals).all()
 
 
 def test_end_to_end_256_device_sweep():

@@ -336,9 +336,20 @@ def test_slow_division_path_with_huge_device_and_record_values():
            "flop_sp_efficiency": 10.0 ** rng.uniform(-2, 2, n),
            "dram_read_bytes": np.floor(10.0 ** rng.uniform(3, 10, n)),
            "dram_write_bytes": np.floor(10.0 ** rng.uniform(3, 10, n))}
-    for origin, dest in ((big, Device.V100), (Device.V100, big), (big, big)):
+    # ordinary limits, but more SMs than the 32-bit model's float ceiling takes
+    # (2^14): the general instantiation, with wave sizes up to 2^25
+    wide = DeviceProperties(name="wide", **dict(Device.V100.as_dict(), num_sms=1 << 20))
+    wide2 = DeviceProperties(name="wide2", **dict(Device.T4.as_dict(), num_sms=(1 << 17) + 3))
+    for origin, dest in ((big, Device.V100), (Device.V100, big), (big, big), (wide2, big)):
         out = wave_scale(KernelRecords.from_numpy(rec), origin, [dest])
         check(rec, origin, [dest], out)
+    # launches that run on such devices, with block counts on both sides of their waves
+    ordinary, _ = synthetic.kernel_records(n, Device.V100, seed=12, metrics_fraction=0.8)
+    ordinary["num_blocks"] = rng.integers(1, 1 << 26, n).astype(np.int32)
+    for origin, dest in ((wide, Device.V100), (Device.V100, wide), (wide, wide2), (wide2, wide)):
+        out = wave_scale(KernelRecords.from_numpy(ordinary), origin, [dest])
+        check(ordinary, origin, [dest], out)
+        assert int((out.status[0] == 0).sum()) > n // 2
 
 
 @pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 130, 255, 256, 257, 258, 386, 1023, 1025, 2050])
