@@ -8,6 +8,7 @@ of a trace and hand them to the GPU in one call each.
 """
 import collections
 import functools
+import itertools
 import logging
 import operator
 import os
@@ -140,6 +141,25 @@ def records_from_kernels(kernels, dest_device, metadata_manager, mode="unified",
     return KernelRecords.from_numpy(rec, device=device or "cuda")
 
 
+_OWN_TIME = operator.attrgetter("_c._run_time_ns")      # this package's MeasuredKernel
+_OWN_BLOCKS = operator.attrgetter("_c._num_blocks")
+_ANY_TIME = operator.attrgetter("run_time_ns")
+_ANY_BLOCKS = operator.attrgetter("num_blocks")
+
+
+def _fingerprint(passes):
+    """What the cached record columns of `passes` were built from, cheaply:
+    the number of kernels, the sums of their times and block counts, and
+    the passes' own times (about 0.15 ms for 900 kernels, a fraction of what
+    converting and uploading them takes)."""
+    kernels = list(itertools.chain.from_iterable(p.kernels for p in passes))
+    try:
+        times, blocks = sum(map(_OWN_TIME, kernels)), sum(map(_OWN_BLOCKS, kernels))
+    except AttributeError:       # kernel objects of another implementation
+        times, blocks = sum(map(_ANY_TIME, kernels)), sum(map(_ANY_BLOCKS, kernels))
+    return (len(kernels), times, blocks, sum(p.run_time_ms for p in passes))
+
+
 class Predictor:
     _RECORD_CACHE_SETS = 8
 
@@ -261,16 +281,20 @@ class Predictor:
 
     def _records_of(self, passes, dest_device, mode):
         """(kernel records of `passes` as columns on the GPU, the kernels'
-        measured times, each pass's overhead).  The last few sets are kept
-        (keyed by the identity of the measured passes, which this package treats
-        as immutable once measured), so that predicting one trace for one
-        destination after another converts and uploads its kernels once.  The
-        register column depends on the destination's architecture only."""
+        measured times, each pass's overhead).  The last few sets are kept, so
+        that predicting one trace for one destination after another converts
+        and uploads its kernels once.  A set is recognised by the identity of
+        its passes AND a fingerprint of what they hold (`_fingerprint`): a pass
+        whose kernels were replaced, added to, or given other times or block
+        counts since is converted afresh, as the reference reads every kernel
+        on every call (predictor.py:111-130).  The register column depends on
+        the destination's architecture only."""
         lut = not isinstance(self._kernel_metadata, NullMetadataManager)
         key = (tuple(id(p) for p in passes), mode, dest_device.compute_capability if lut else None,
                torch.cuda.current_device())
+        mark = _fingerprint(passes)
         hit = self._record_cache.get(key)
-        if hit is not None:
+        if hit is not None and hit[4] == mark:
             self._record_cache.move_to_end(key)
             return hit[:3]
         kernels = [k for p in passes for k in p.kernels]
@@ -279,14 +303,16 @@ class Predictor:
         measured_ns = [k.run_time_ns for k in kernels]
         overheads_ns = [self._overhead_ns(p) for p in passes]
         # the passes stay alive with their ids
-        self._record_cache[key] = (rec, measured_ns, overheads_ns, list(passes))
+        self._record_cache[key] = (rec, measured_ns, overheads_ns, list(passes), mark)
+        self._record_cache.move_to_end(key)
         while len(self._record_cache) > self._RECORD_CACHE_SETS:
             self._record_cache.popitem(last=False)
         return rec, measured_ns, overheads_ns
 
     def clear_record_cache(self):
-        """Forget the cached kernel-record columns (after changing a measured
-        kernel in place)."""
+        """Forget the cached kernel-record columns (only needed after a change
+        the fingerprint cannot see, such as editing a kernel's metrics or
+        launch configuration in place while its time and block count stay)."""
         self._record_cache.clear()
 
     @staticmethod

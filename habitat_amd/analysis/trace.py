@@ -4,6 +4,7 @@ prediction for another (analyzer/habitat/analysis/trace.py:5-51).
 Unlike the reference, importing this module needs no data files: the default
 predictor is built on first use.
 """
+from habitat_amd.analysis.operation import MeasuredOperation
 from habitat_amd.analysis.predictor import Predictor
 
 
@@ -49,7 +50,20 @@ class Trace:
         if dest_device.name == self.device.name:
             return self
         predictor = predictor if predictor is not None else Trace.default_predictor()
-        return Trace(dest_device, predictor.predict_operations(self._operations, dest_device))
+        # Each operation keeps the contract of its own to_device (trace.py:46-49
+        # maps it over the operations): one already measured on the destination
+        # is returned as it is and a predicted one refuses; the measured ones
+        # that do need predicting go to the GPU together.
+        operations = list(self._operations)
+        batch = [i for i, op in enumerate(operations)
+                 if isinstance(op, MeasuredOperation) and op.device.name != dest_device.name]
+        for i, op in enumerate(operations):
+            if not isinstance(op, MeasuredOperation) or op.device.name == dest_device.name:
+                operations[i] = op.to_device(dest_device, predictor)
+        predicted = predictor.predict_operations([operations[i] for i in batch], dest_device)
+        for i, op in zip(batch, predicted):
+            operations[i] = op
+        return Trace(dest_device, operations)
 
     def to_devices(self, dest_devices, predictor=None, device_features=None):
         """Predicted run time [ms] of the whole trace on each device of a sweep,

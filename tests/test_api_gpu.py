@@ -269,6 +269,67 @@ def test_bmm_lstm_and_every_call_form_against_hand_listed_features():
         assert abs(got.run_time_ms - w) <= tol, case[:2]
 
 
+def test_changed_kernels_are_seen_without_clearing_the_record_cache():
+    """The predictor keeps the GPU-resident record columns of the passes it has
+    seen; a pass whose kernels changed since (a time edited in place, a kernel
+    replaced, one appended) must be converted afresh, as the reference reads
+    every kernel on every call (predictor.py:111-130)."""
+    origin, dest = Device.V100, Device.T4
+    ops = [o for o in synthetic.resnet50_trace(origin, batch=8, seed=9).operations
+           if o.name not in ("conv2d", "linear")][:12]
+    trace = Trace(origin, ops)
+    predictor = Predictor(mlp_predictors={})
+
+    def oracle_total():
+        return opred.trace_ms([oracle_operation_ms(op, dest, {}) for op in ops])
+
+    first = trace.to_device(dest, predictor).run_time_ms
+    assert first == pytest.approx(oracle_total(), rel=1e-6)
+    assert trace.to_device(dest, predictor).run_time_ms == first          # served from the cache
+    # 1. a kernel's time edited in place (and its pass, so that the overhead stays)
+    victim = ops[3].forward.kernels[0]
+    victim._c._run_time_ns += 7_000_000
+    ops[3].forward._run_time_ms += 7.0
+    second = trace.to_device(dest, predictor).run_time_ms
+    assert second == pytest.approx(oracle_total(), rel=1e-6) and second > first + 1.0
+    # 2. a kernel replaced by one with another launch size
+    old = ops[5].forward.kernels[0]
+    ops[5].forward.kernels[0] = make_kernel(origin, num_blocks=old.num_blocks * 3 + 1,
+                                            t_ns=old.run_time_ns, name="other")
+    third = trace.to_device(dest, predictor).run_time_ms
+    assert third == pytest.approx(oracle_total(), rel=1e-6)
+    # 3. a kernel appended
+    ops[7].forward.kernels.append(make_kernel(origin, num_blocks=12345, t_ns=2_500_000, name="more"))
+    fourth = trace.to_device(dest, predictor).run_time_ms
+    assert fourth == pytest.approx(oracle_total(), rel=1e-6) and fourth != third
+
+
+def test_trace_to_device_keeps_each_operation_s_own_contract():
+    """trace.py:46-49 maps operation.to_device over the operations: one measured
+    on the destination already comes back as it is (operation.py:82-85), a
+    predicted one refuses (operation.py:137)."""
+    from habitat_amd.analysis.operation import MeasuredOperation
+    origin, dest = Device.V100, Device.T4
+    ops = [o for o in synthetic.resnet50_trace(origin, batch=8, seed=9).operations
+           if o.name not in ("conv2d", "linear")][:6]
+    at_home = [o for o in synthetic.resnet50_trace(dest, batch=8, seed=9).operations
+               if o.name not in ("conv2d", "linear")][0]
+    assert isinstance(at_home, MeasuredOperation) and at_home.device is dest
+    predictor = Predictor(mlp_predictors={})
+    mixed = Trace(origin, ops[:3] + [at_home] + ops[3:])
+    out = mixed.to_device(dest, predictor)
+    assert out.operations[3] is at_home
+    for i in (0, 1, 2, 4, 5, 6):
+        assert out.operations[i].device is dest and out.operations[i] is not mixed.operations[i]
+        want = oracle_operation_ms(mixed.operations[i], dest, {})
+        assert out.operations[i].run_time_ms == pytest.approx(want, rel=1e-6)
+    # a predicted trace cannot be predicted from
+    with pytest.raises(RuntimeError, match="predicted operation"):
+        out.to_device(Device.P100, predictor)
+    # ... but still answers for the device it is on
+    assert out.to_device(dest, predictor) is out
+
+
 def test_predictor_with_a_caller_supplied_strategy_and_pass_through_ops():
     from habitat_amd.analysis.arguments import Arguments
     from habitat_amd.analysis.operation import MeasuredOperation
