@@ -11,6 +11,8 @@ LIB_PATH = os.path.join(HERE, "lib", "libhabitat_mi.so")
 
 ABI_VERSION = 101   # HBT_VERSION of include/habitat_mi.h this binding was written for
 
+MLP_STATIC_MAX_ROWS = 1024   # HBT_MLP_STATIC_MAX_ROWS
+
 HBT_OK, HBT_EINVAL, HBT_ESPEC, HBT_EHIP, HBT_ENOMEM, HBT_EALIGN, HBT_ESIZE = 0, -1, -2, -3, -4, -5, -6
 ST_OK, ST_ORIGIN_WAVE_ZERO, ST_DEST_WAVE_ZERO, ST_BAD_GAMMA, ST_ZERO_BLOCKS = 0, 1, 2, 3, 4
 
@@ -62,6 +64,7 @@ _SIGNATURES = {
                             C.POINTER(C.c_int)]),
     "hbt_mlp_forward": (C.c_int, [_P, _P, C.c_int64, _P, _P]),
     "hbt_mlp_destroy": (None, [_P]),
+    "hbt_mlp_forward_static": (C.c_int, [_P, _P, C.c_int64, _P, _P]),
     "hbt_local_device_spec": (C.c_int, [C.c_int, C.POINTER(DeviceSpec), C.c_char_p, C.c_size_t]),
     "hbt_measure_fp32_fma_gflops": (C.c_int, [C.c_int, C.POINTER(C.c_double)]),
     "hbt_measure_fp32_mfma_gflops": (C.c_int, [C.c_int, C.POINTER(C.c_double)]),

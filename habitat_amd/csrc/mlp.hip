@@ -32,6 +32,7 @@
 
 #include <cstdint>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -699,14 +700,52 @@ size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 }  // namespace
 }  // namespace hbt
 
+// Scratch memory of hbt_mlp_forward_static: the per-layer path's two buffers
+// for up to HBT_MLP_STATIC_MAX_ROWS rows, part of the code object (each GPU the
+// library runs on holds its own copy until the process ends).  In host code
+// this name is only a handle for hipGetSymbolAddress: kernels and copies get
+// the per-device address kept in static_scratch_of().
+constexpr int kStaticMaxRows = HBT_MLP_STATIC_MAX_ROWS;
+constexpr size_t kStaticFloats = (size_t)kStaticMaxRows * hbt::kWidth;  // each of the two
+static_assert((size_t)hbt::kSplit * hbt::kRows * hbt::kWidth <= kStaticFloats &&
+                  2 * (size_t)hbt::kHalfKMaxTiles * hbt::kRows * hbt::kWidth <= kStaticFloats &&
+                  kStaticMaxRows % hbt::kRows == 0 && kStaticMaxRows <= hbt::kLayerMaxRows,
+              "the K-partials of the small shapes and the padded rows fit the static scratch");
+static __device__ __align__(256) float scratch[2 * kStaticFloats];
+
 namespace {
 
-// One launch per layer for n <= kLayerMaxRows rows, through the handle's two
-// scratch buffers.
+// The device address of `scratch` on the current device, looked up once per
+// device (nullptr and *rc set when the runtime refuses).
+constexpr int kMaxDevices = 64;
+float* static_scratch_of(int device, int* rc) {
+  static std::mutex lock;
+  static float* address[kMaxDevices] = {};
+  *rc = HBT_OK;
+  if (device < 0 || device >= kMaxDevices) {
+    *rc = HBT_ESIZE;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> guard(lock);
+  if (address[device] == nullptr) {
+    float* ptr = nullptr;
+    if (hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess ||
+        ptr == nullptr) {
+      (void)hipGetLastError();
+      *rc = HBT_EHIP;
+      return nullptr;
+    }
+    address[device] = ptr;
+  }
+  return address[device];
+}
+
+// One launch per layer for n <= kLayerMaxRows rows, through two buffers of
+// activations or K-partials (each at least max(n rounded up to 32, kSplit * 32)
+// x kWidth floats): the handle's, or the library's static ones.
 int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* out,
-                   hipStream_t stream) {
+                   float* const buffers[2], hipStream_t stream) {
   using namespace hbt;
-  // one launch per layer, through the handle's two scratch buffers
   const int m_tiles = (int)((n + kRows - 1) / kRows);
   const bool split_k = n <= kSplitMaxRows;
   // with a few m-tiles the eight-wave shape splits K in two as well
@@ -727,7 +766,7 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
     l.p_in = p_in;
     l.bias_in = (layer == 0) ? nullptr : mlp->bias + (size_t)(layer - 1) * kWidth;
     l.bias_out = mlp->bias + (size_t)layer * kWidth;
-    l.p_out = mlp->scratch[layer & 1];
+    l.p_out = buffers[layer & 1];
     const dim3 grid(kWidth / 32, (unsigned)l.splits, (unsigned)m_tiles);
     if (layer == 0 && split_k)
       hipLaunchKernelGGL((mlp_layer_kernel<true, 0, true, 4, false, 0>), grid, dim3(256), 0,
@@ -954,11 +993,37 @@ int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* 
   while (done < n) {
     const int64_t rows = n - done < kLayerMaxRows ? n - done : kLayerMaxRows;
     const int rc = forward_layers(mlp, raw_features + done * mlp->in_features, rows, out + done,
-                                  stream);
+                                  mlp->scratch, stream);
     if (rc != HBT_OK) return rc;
     done += rows;
   }
   return HBT_OK;
+}
+
+int hbt_mlp_forward_static(hbt_mlp* mlp, const double* raw_features, int64_t n, float* out,
+                           void* hip_stream) {
+  using namespace hbt;
+  if (mlp == nullptr || n < 0) return HBT_EINVAL;
+  if (n > kStaticMaxRows) return HBT_ESIZE;
+  if (n == 0) return HBT_OK;
+  if (raw_features == nullptr || out == nullptr) return HBT_EINVAL;
+  if ((reinterpret_cast<uintptr_t>(raw_features) % 8) != 0 ||
+      (reinterpret_cast<uintptr_t>(out) % 4) != 0)
+    return HBT_EALIGN;
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    return HBT_EHIP;
+  }
+  if (device != mlp->device) return HBT_EINVAL;
+  int rc = HBT_OK;
+  float* base = static_scratch_of(device, &rc);
+  if (base == nullptr) return rc;
+  // Every value a layer reads was written by the layer before it in this call
+  // (rows past n within the last 32-row tile included), so nothing needs
+  // clearing between calls.
+  float* const buffers[2] = {base, base + kStaticFloats};
+  return forward_layers(mlp, raw_features, n, out, buffers, static_cast<hipStream_t>(hip_stream));
 }
 
 void hbt_mlp_destroy(hbt_mlp* mlp) {

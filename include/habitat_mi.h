@@ -8,7 +8,8 @@
  * and the call returns without synchronising.  Functions return 0 or a
  * negative HBT_E* code; hbt_strerror() names it.  There is no global state and
  * no CPU fallback: without a GPU the compute entry points return HBT_EHIP.
- * Only the two *_create calls allocate device memory.
+ * Only the two *_create calls allocate device memory (and the calibration
+ * calls at the end, which say so).
  *
  * Each entry point cites the reference interface it stands in for
  * (paths relative to the reference tree).
@@ -263,6 +264,26 @@ hbt_mlp *hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
 int hbt_mlp_forward(hbt_mlp *mlp, const double *raw_features, int64_t n, float *out,
                     void *hip_stream);
 void hbt_mlp_destroy(hbt_mlp *mlp);
+
+/*
+ * hbt_mlp_forward for callers that cannot allocate device memory or tolerate a
+ * library that does: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  The same
+ * per-layer kernels as hbt_mlp_forward runs for such row counts (and therefore
+ * bit-identical results), but their scratch (activations or partial sums
+ * between the layer launches) lives in a static device array of the library, 2
+ * x 4 MiB per GPU for the life of the process, not in memory of the handle; the
+ * call allocates and frees nothing.  n > HBT_MLP_STATIC_MAX_ROWS returns
+ * HBT_ESIZE.  All calls on one GPU share that array, whatever handle or stream
+ * they use: calls that overlap on one GPU race; calls that follow each other on
+ * one stream, or are otherwise ordered, are fine (nothing is carried over from
+ * one call to the next).  The first call on a device looks the array's address
+ * up (hipGetSymbolAddress), so make it outside any graph capture.  Must be
+ * called with the device of hbt_mlp_create current.
+ */
+#define HBT_MLP_STATIC_MAX_ROWS 1024
+int hbt_mlp_forward_static(hbt_mlp *mlp, const double *raw_features, int64_t n, float *out,
+                           void *hip_stream);
 
 /*
  * Calibration of the GPU this process runs on.  Not part of the prediction
