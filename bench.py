@@ -18,6 +18,7 @@ inputs resident in HBM.  Prints ONE JSON line:
                 large_16M: at 16 M records
   mlp           the fused MFMA MLP (configs[2], conv2d, 1 M rows): rows/s, its
                 roofline against fp32 MFMA peak and a torch-CPU fp32 baseline
+  scalar_strategy  the reference's one-kernel strategy call through the same kernel
   sweep         configs[4]: one ResNet-50-shaped trace predicted for 256 devices
                 (fused per-pass sums + MLP rows + ratio kernel), eager and as a
                 replayed HIP graph, next to the per-device CPU path
@@ -130,7 +131,7 @@ def tile_records(rec, n):
 
 def mlp_bench(args):
     """configs[2] (and the other kinds of configs[3], one step each): the fused
-    MLP at full size, the per-layer path (up to 6400 rows, 4096 at a time), and a torch CPU baseline."""
+    MLP at full size, the per-layer path (up to 7168 rows), and a torch CPU baseline."""
     import torch
     from habitat_amd import synthetic
     from habitat_amd.analysis.mlp.mlp import RuntimePredictor
@@ -172,10 +173,10 @@ def mlp_bench(args):
                       "the first %d rows, %d torch threads" % (m, threads)}
     # few rows: the reference's own call pattern is one row per call (mlp.py:252-267)
     few = {}
-    for rows in (1, 108, 512, 4096):
+    for rows in (1, 48, 108, 512, 1536, 4096, 5911):
         xs = xg[:rows].contiguous()
         ys = torch.empty(rows, dtype=torch.float32, device="cuda")
-        _, f_launch = time_steps(lambda: rp.predict_batch(xs, out=ys), 50, 5)
+        _, f_launch = time_steps(lambda: rp.predict_batch(xs, out=ys), 200, 50)
         few["rows_%d_us" % rows] = f_launch * 1e3
     if not args.no_cpu:
         from oracle import mlp as omlp
@@ -185,8 +186,8 @@ def mlp_bench(args):
         for i in range(20):
             omlp.forward_fp32(sd, x[i:i + 1], mu, sigma)
         few["cpu_rows_1_us"] = (time.perf_counter() - t0) / 20 * 1e6
-    few["note"] = ("up to 6400 rows, 4096 at a time: one launch per layer over the whole GPU "
-                   "(mlp_layer_kernel); "
+    few["note"] = ("up to 7168 rows: one launch per layer over the whole GPU "
+                   "(mlp_layer_kernel up to 128 rows, mlp_layer_tile_kernel above); "
                    "cpu_rows_1_us: torch CPU fp32, batch 1, as the reference predicts")
     mlp["few_rows"] = few
     others = {}
@@ -235,7 +236,7 @@ def sweep_bench(args, origin):
     call = plan.prepare(devices, device_features)
     torch.cuda.synchronize()
     prepare_ms = (time.perf_counter() - t0) * 1e3
-    eager_wall, eager_gpu = time_steps(call.launch, 50, 5)
+    eager_wall, eager_gpu = time_steps(call.launch, 200, 50)
     totals = call.launch().total_ms
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
@@ -247,7 +248,7 @@ def sweep_bench(args, origin):
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         captured = call.launch()
-    graph_wall, graph_gpu = time_steps(graph.replay, 50, 5)
+    graph_wall, graph_gpu = time_steps(graph.replay, 200, 50)
     torch.cuda.synchronize()
     same = bool(torch.allclose(captured.total_ms, totals, rtol=1e-12, atol=0))
     n_kernels = len(plan.kernels)
@@ -422,13 +423,52 @@ def main():
     if not args.no_cpu:
         attempt("cpu_baseline", cpu_section)
 
+    # ---------------- the reference's plug point: one kernel per call ----------------
+    def scalar_section():
+        from habitat_amd.analysis.kernels import KernelInstance, MeasuredKernel
+        from habitat_amd.analysis.wave_scaling.metadata import NullMetadataManager
+        from habitat_amd.analysis.wave_scaling.unified import unified_wave_scaling
+        m = 2000
+        kernels = []
+        for i in range(m):
+            f = {k: v[i].item() for k, v in rec.items()}
+            args_ = ("k", f["num_blocks"], f["block_size"], f["dynamic_smem"], f["static_smem"],
+                     f["regs_per_thread"], int(f["run_time_ns"]))
+            with_metrics = KernelInstance(*args_, [
+                ("flop_sp_efficiency", f["flop_sp_efficiency"]),
+                ("dram_read_bytes", f["dram_read_bytes"]),
+                ("dram_write_bytes", f["dram_write_bytes"])])
+            kernels.append(MeasuredKernel(KernelInstance(*args_), [with_metrics], origin))
+        mm = NullMetadataManager()
+        skipped = 0
+        for k in kernels[:200]:
+            try:
+                unified_wave_scaling(k, origin, dest, mm)
+            except ZeroDivisionError:
+                pass
+        t0 = time.perf_counter()
+        for k in kernels:
+            try:
+                unified_wave_scaling(k, origin, dest, mm)
+            except ZeroDivisionError:      # destination occupancy 0: the reference raises too
+                skipped += 1
+        dt = time.perf_counter() - t0
+        return {"scalar_strategy_us_per_kernel": dt / m * 1e6, "kernels": m, "raised": skipped,
+                "what": "unified_wave_scaling(kernel, origin, dest, manager), the reference's "
+                        "strategy signature (predictor.py:116-124): per call one 64-byte upload, "
+                        "one launch, one 24-byte read-back and a wait"}
+
+    attempt("scalar_strategy", scalar_section)
+
     # ---------------- the same kernel beyond the last-level cache ----------------
     def large_section(n_records=None):
         big = KernelRecords.from_numpy(tile_records(rec, n_records or args.large_records))
         big_out = WaveScaleOutput(big.n, 1, big.device, waves=False, status=True)
         big_call = WaveScaleCall(big, origin, dest, big_out)
-        steps = max(5, min(args.steps, 40))
-        b_wall, b_launch = time_steps(big_call, steps, min(args.warmup, 20))
+        # launch counts of this section's own, whatever --steps / --warmup say
+        # (about 60 ms of launches at either size)
+        steps = 80 if big.n > 32_000_000 else 300
+        b_wall, b_launch = time_steps(big_call, steps, steps // 4)
         b_ach = BYTES_PER_RECORD * big.n / (b_launch * 1e-3) / 1e9
         return {"records": big.n, "steps": steps, "ms_per_step": b_wall,
                 "value": big.n / (b_wall * 1e-3), "unit": "records/s",
@@ -442,7 +482,9 @@ def main():
                  if name != origin.name and not name.startswith("MI355X")]
         m_out = WaveScaleOutput(records.n, len(dests), records.device, waves=False, status=True)
         m_call = WaveScaleCall(records, origin, dests, m_out)
-        m_wall, m_launch = time_steps(m_call, max(args.steps // 4, 5), max(args.warmup // 4, 2))
+        # launch counts of this section's own: a short run after a cold start
+        # reads 60 % high (the kernel instantiation is loaded on first use)
+        m_wall, m_launch = time_steps(m_call, 500, 200)
         per_record = 52 + 17 * len(dests)     # the record is read once per launch
         gbs = per_record * records.n / (m_launch * 1e-3) / 1e9
         return {"destinations": [d.name for d in dests], "launch_us": m_launch * 1e3,
@@ -482,7 +524,7 @@ def main():
                "fp32_vector_fma_TFLOPs": m["fp32_fma_gflops"] / 1e3}
         # yardstick for wave scaling: its loads and stores without the arithmetic
         out["record_stream_GBps_at_%d_records" % args.records] = device_info.record_stream_gbps(
-            args.records, args.warmup, args.steps)
+            args.records, 500, 2000)
         out["record_stream_GBps_at_%d_records" % args.large_records] = (
             device_info.record_stream_gbps(args.large_records, 20, 40))
         # yardstick for the MLP: the vendor library's fp32 GEMM (+ bias) on one hidden

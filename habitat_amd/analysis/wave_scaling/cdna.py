@@ -33,6 +33,10 @@ def native_description(device):
     if major == _HIP_GFX9_MAJOR:
         props = device.as_dict()
         props["compute_major"] = CDNA_MAJOR
+        # hipDeviceProp_t counts the 256 architectural VGPRs per lane and SIMD;
+        # gfx942 and gfx950 (9.4, 9.5) allocate from a unified file of 512
+        if minor >= 4 and props["regs_per_multiprocessor"] == 4 * 256 * props["warp_size"]:
+            props["regs_per_multiprocessor"] *= 2
         return DeviceProperties(name=device.name, **props)
     if device.name + "_cdna" in Device.names():
         return getattr(Device, device.name + "_cdna")

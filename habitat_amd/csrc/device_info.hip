@@ -164,10 +164,17 @@ int hbt_local_device_spec(int device, hbt_device_spec* out, char* name, size_t n
   out->smem_per_block = (int64_t)p.sharedMemPerBlock;
   out->smem_per_sm = (int64_t)p.maxSharedMemoryPerMultiProcessor;
   out->smem_per_block_optin = (int64_t)p.sharedMemPerBlockOptin;
-  // memoryClockRate is in kHz, double data rate; bus width in bits
-  out->mem_bandwidth_gb = 2.0 * p.memoryClockRate * 1e3 * (p.memoryBusWidth / 8.0) / 1e9;
+  // memoryClockRate is in kHz, the bus width in bits.  HBM2/2e (up to gfx90a)
+  // moves two bits per pin and reported clock, HBM3/3E (gfx942, gfx950) four:
+  // MI300X reports 1300 MHz x 8192 bit for 5.3 TB/s, MI355X 2000 MHz x 8192 bit
+  // for 8 TB/s.
+  const double bits_per_clock = (p.major == 9 && p.minor >= 4) ? 4.0 : 2.0;
+  out->mem_bandwidth_gb =
+      bits_per_clock * p.memoryClockRate * 1e3 * (p.memoryBusWidth / 8.0) / 1e9;
   out->base_clock_mhz = p.clockRate / 1e3;
-  // vector fp32: 64 lanes x 2 FLOP per CU and clock
+  // vector fp32 as an ordinary kernel reaches it: 64 lanes x one FMA (2 FLOP)
+  // per CU and clock.  The published fp32 figure (157.3 TFLOP/s on MI355X) is
+  // twice that: it counts packed fp32 or the matrix cores.
   out->peak_gflops = p.multiProcessorCount * (p.clockRate / 1e6) * 128.0;
   if (name != nullptr && name_len > 0) {
     std::strncpy(name, p.name, name_len - 1);

@@ -309,12 +309,10 @@ constexpr int kSplit = 8;            // K-partials per hidden layer, up to kSpli
 // 16 / 24 / 32 rows: split 39 44 52 61 71 us (the partials' traffic grows with
 // the rows), whole K 57 us at any of them.
 constexpr int kSplitMaxRows = 20;
-constexpr int kLayerMaxRows = 4096;  // largest batch that takes this path in one pass
-// Largest batch that takes this path in two passes (4096 rows, then the rest).
-// Measured, two passes against one round of the fused kernel (940 us): 4200
-// rows 612 us, 5120 712, 5686 841, 6144 846, 6656 913, 7168 979.
-constexpr int kLayerTwoPassRows = kLayerMaxRows + 2304;
-constexpr int kManyTiles = 32;       // m-tiles from which a workgroup takes two n-tiles (NT)
+// Largest batch that takes this path (224 m-tiles: 7 steps of the tile kernel).
+// Measured against one round of the fused kernel (940 us whatever it holds up to
+// 8192 rows): 6144 rows 744 us, 7168 rows 862, 7296 rows 975.
+constexpr int kLayerMaxRows = 7168;
 // m-tiles up to which the eight-wave shape splits K over two workgroups (128
 // workgroups or fewer per layer would leave half the compute units idle).
 // Measured per forward at 32 / 64 / 128 / 256 rows: 49 52 58 82 us against 57 57
@@ -555,6 +553,112 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
   }
 }
 
+// One hidden layer with a wave owning ONE output tile (32 rows x 32 outputs) for
+// 1 / KS of K: no loop over tiles, accumulators in place for the wave's whole
+// run of k-groups, fragments through a ring of SLOTS register slots (loads
+// SLOTS - 1 k-groups ahead of their MFMAs, one 16-byte buffer load per lane and
+// fragment, 1 KiB of contiguous memory per wave), no LDS staging.  A workgroup
+// is four waves:
+//   KS = 1   2 m-tiles x 2 n-tiles, no reduction, no barrier
+//   KS = 2   1 m-tile x 2 n-tiles, two halves of K
+//   KS = 4   1 m-tile x 1 n-tile, four quarters of K
+// With KS > 1 the waves of a tile add their accumulators through LDS in wave
+// order, each finishing 16 / KS of the tile's registers.  A tile for the whole
+// of K is 13.7 us of one SIMD's matrix core, so a layer takes that times the
+// tiles per SIMD, rounded up: KS trades a finer rounding (1024 / KS rows per
+// step) against shorter runs per wave.  Activations in and out are stored by
+// k-group (km_index); bias and ReLU are applied on the way out.
+// Measured per forward at 4096 rows with KS = 1: a wave owning 2 x 2 tiles 526
+// us, 1 x 2 tiles 514, one tile 501 (8 ring slots: 503); workgroups numbered
+// m-tile first instead of n-tile first: no difference.
+template <int KS, int SLOTS>
+__global__ __launch_bounds__(256) void mlp_layer_tile_kernel(const LayerArgs a) {
+  static_assert(KS == 1 || KS == 2 || KS == 4, "four waves per workgroup");
+  constexpr int kGroups = kWidth / 8 / KS;  // per wave
+  static_assert(kGroups % SLOTS == 0, "the ring turns a whole number of times");
+  __shared__ float red[KS > 1 ? 4 : 1][16][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int m = lane & 31, h = lane >> 5;
+  const int m_tiles = a.m_pad / kRows;
+  // wave -> (part of K, n-tile, m-tile)
+  const int k_part = wave % KS;
+  const int n_tile = KS == 4 ? (int)blockIdx.x : (int)blockIdx.x * 2 + (KS == 2 ? wave >> 1 : wave & 1);
+  const int m_tile = KS == 1 ? (int)blockIdx.y * 2 + (wave >> 1) : (int)blockIdx.y;
+  if (m_tile >= m_tiles) return;  // KS = 1 only (no barrier there): an odd number of m-tiles
+
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(a.w_stream), 0, 4 * a.groups_total * (8 * 64 * 16), 0x00020000);
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(a.p_in), 0, a.m_pad * (kWidth * 4), 0x00020000);
+  const int first = k_part * kGroups;  // the wave's first k-group of the layer
+  const int w_lane_bytes = ((n_tile & 7) * 64 + lane) * 16;
+  const int w_base_bytes = ((n_tile >> 3) * a.groups_total + a.g0 + first) * (8 * 64 * 16);
+  const int x_lane_bytes = m_tile * (kWidth * kRows * 4) + m * 32 + 16 * h;
+  const int x_base_bytes = first * (kRows * 32);
+
+  f32x4 w[SLOTS], x[SLOTS];
+  auto load = [&](int slot, int group) {
+    w[slot] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+        w_rsrc, w_lane_bytes, w_base_bytes + group * (8 * 64 * 16), 0));
+    x[slot] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+        x_rsrc, x_lane_bytes, x_base_bytes + group * (kRows * 32), 0));
+  };
+
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+  for (int s = 0; s < SLOTS - 1; ++s) load(s, s);
+  for (int j = 0; j < kGroups; j += SLOTS) {
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) {
+      // past the wave's last group the last one is fetched again (unused)
+      const int ahead = j + s + SLOTS - 1;
+      load((s + SLOTS - 1) % SLOTS, ahead < kGroups ? ahead : kGroups - 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[s][e], x[s][e], acc, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // accumulator register 4g + e of lane (m, h) is output n = 8g + 4h + e of row m
+  auto finish = [&](int g, const f32x4 sum) {
+    const int n0 = n_tile * 32 + 8 * g + 4 * h;
+    const f32x4 bias = *reinterpret_cast<const f32x4*>(a.bias_out + n0);
+    f32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = relu(sum[e] + bias[e]);
+    *reinterpret_cast<f32x4*>(a.p_out + km_index(m_tile, n0 >> 3, m, 4 * h)) = o;
+  };
+  if constexpr (KS == 1) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) finish(g, f32x4{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]});
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[wave][r][lane] = acc[r];
+    __syncthreads();
+    // the KS waves of a tile are wave0 .. wave0 + KS - 1; this one finishes the
+    // register groups g0 .. g0 + 4 / KS - 1, adding the parts of K in wave order
+    const int wave0 = wave - k_part;
+#pragma unroll
+    for (int i = 0; i < 4 / KS; ++i) {
+      const int g = k_part * (4 / KS) + i;
+      f32x4 sum;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float v = red[wave0][4 * g + e][lane];
+#pragma unroll
+        for (int p = 1; p < KS; ++p) v += red[wave0 + p][4 * g + e][lane];
+        sum[e] = v;
+      }
+      finish(g, sum);
+    }
+  }
+}
+
 struct LastArgs {
   const float* p_in;     // m_pad x kWidth activations, or S_IN such blocks of K-partials
   const float* bias_in;  // [kWidth], bias of the last hidden layer (with partials)
@@ -740,6 +844,27 @@ float* static_scratch_of(int device, int* rc) {
   return address[device];
 }
 
+// Into how many parts mlp_layer_tile_kernel splits K for a batch of m_tiles
+// m-tiles.  A layer is 32 m_tiles output tiles on 1024 SIMDs and takes
+// ceil(32 m_tiles KS / 1024) steps of 13.7 / KS us: the finest split is never
+// worse by that count, but a wave's run gets shorter (a run of 32 k-groups is 3.4
+// us, next to about a microsecond until its first fragments arrive) and all
+// workgroups should be resident at once (8 per compute unit), so the coarsest
+// split among the cheapest is taken, KS = 2 up to 4096 rows and KS = 4 up to 2048.
+// Measured per forward, as (rows: us with KS = 1 / 2 / 4; the 8-wave whole-K
+// kernel this path replaced): 512: 156 / 99 / 99; 103.  1280: 263 / 208 / 183;
+// 225.  2560: 382 / 330 / 427; 361.  4096: 506 / 512 / 598; 559.  6144: 744 / 862
+// / 822; 821.
+int tile_k_parts(int m_tiles) {
+  int best = 1, best_cost = (m_tiles + 31) / 32 * 4;  // in quarter steps
+  if (m_tiles <= 128 && (m_tiles + 15) / 16 * 2 < best_cost) {
+    best = 2;
+    best_cost = (m_tiles + 15) / 16 * 2;
+  }
+  if (m_tiles <= 64 && (m_tiles + 7) / 8 < best_cost) best = 4;
+  return best;
+}
+
 // One launch per layer for n <= kLayerMaxRows rows, through two buffers of
 // activations or K-partials (each at least max(n rounded up to 32, kSplit * 32)
 // x kWidth floats): the handle's, or the library's static ones.
@@ -759,6 +884,7 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
   l.m_pad = m_tiles * kRows;
   bool partials = false;
   const float* p_in = nullptr;
+  const int tile_ks = tile_k_parts(m_tiles);
   for (int layer = 0; layer <= mlp->hidden; ++layer) {
     l.g0 = (layer == 0) ? 0 : mlp->in_padded / 8 + (layer - 1) * (kWidth / 8);
     l.kg = (layer == 0) ? mlp->in_padded / 8 : kWidth / 8;
@@ -780,12 +906,15 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
     else if (ks == 2)
       hipLaunchKernelGGL((mlp_layer_kernel<false, 2, false, 8, true, 2, 1, true, 2>), grid,
                          dim3(512), 0, stream, l);
-    else if (!split_k && m_tiles < kManyTiles)
-      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 2, 1, true>), grid, dim3(512),
-                         0, stream, l);
+    else if (!split_k && tile_ks == 1)
+      hipLaunchKernelGGL((mlp_layer_tile_kernel<1, 4>),
+                         dim3(kWidth / 64, (unsigned)((m_tiles + 1) / 2)), dim3(256), 0, stream, l);
+    else if (!split_k && tile_ks == 2)
+      hipLaunchKernelGGL((mlp_layer_tile_kernel<2, 4>), dim3(kWidth / 64, (unsigned)m_tiles),
+                         dim3(256), 0, stream, l);
     else if (!split_k)
-      hipLaunchKernelGGL((mlp_layer_kernel<false, 0, true, 8, true, 0, 2, true>),
-                         dim3(kWidth / 64, 1, (unsigned)m_tiles), dim3(512), 0, stream, l);
+      hipLaunchKernelGGL((mlp_layer_tile_kernel<4, 4>), dim3(kWidth / 32, (unsigned)m_tiles),
+                         dim3(256), 0, stream, l);
     else if (partials)
       hipLaunchKernelGGL((mlp_layer_kernel<false, kSplit, false, 4, false, 0>), grid, dim3(256),
                          0, stream, l);
@@ -977,27 +1106,19 @@ int hbt_mlp_forward(hbt_mlp* mlp, const double* raw_features, int64_t n, float* 
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
   // The fused kernel keeps every compute unit busy for whole rounds of
   // 32 rows x compute units (about 0.94 ms each); what is left over after the
-  // last whole round would cost another one.  Leftover rows go through the
-  // per-layer path instead where that takes less: up to kLayerMaxRows in one
-  // pass, up to kLayerTwoPassRows in two (the passes share the scratch buffers
-  // and follow each other on the stream).
+  // last whole round would cost another one.  Up to kLayerMaxRows leftover rows
+  // go through the per-layer path instead, which takes less for them.
   const int64_t round_rows = (int64_t)kRows * mlp->compute_units;
   const int64_t leftover = n % round_rows;
-  if (leftover == 0 || leftover > kLayerTwoPassRows)
+  if (leftover == 0 || leftover > kLayerMaxRows)
     return forward_fused(mlp, raw_features, n, out, stream);
-  int64_t done = n - leftover;
+  const int64_t done = n - leftover;
   if (done > 0) {
     const int rc = forward_fused(mlp, raw_features, done, out, stream);
     if (rc != HBT_OK) return rc;
   }
-  while (done < n) {
-    const int64_t rows = n - done < kLayerMaxRows ? n - done : kLayerMaxRows;
-    const int rc = forward_layers(mlp, raw_features + done * mlp->in_features, rows, out + done,
-                                  mlp->scratch, stream);
-    if (rc != HBT_OK) return rc;
-    done += rows;
-  }
-  return HBT_OK;
+  return forward_layers(mlp, raw_features + done * mlp->in_features, leftover, out + done,
+                        mlp->scratch, stream);
 }
 
 int hbt_mlp_forward_static(hbt_mlp* mlp, const double* raw_features, int64_t n, float* out,

@@ -250,15 +250,15 @@ hbt_mlp *hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
  * through the network; out[n] receives the fp32 predictions.  Must be called
  * with the device of hbt_mlp_create current.  Large batches go through one
  * fused kernel that runs the whole network with activations on-chip, in whole
- * rounds of 32 rows per compute unit; up to 6400 rows (a single prediction,
+ * rounds of 32 rows per compute unit; up to 7168 rows (a single prediction,
  * the operations of one trace, a trace for some devices, or what is left over
  * after the last whole round) each layer is one launch spread over the whole
- * GPU, at most 4096 rows at a time, with activations or partial sums in a
- * scratch buffer that belongs to the handle (2 x 16 MiB, allocated by
- * hbt_mlp_create): calls on ONE handle must therefore not overlap, on any
- * streams; different handles are independent.
- * Results are reproducible for a given n and position of the row; the paths
- * (up to 20 rows, up to 6400 in passes of at most 4096, above) sum in different orders and agree to fp32
+ * GPU, with activations or partial sums in a scratch buffer that belongs to
+ * the handle (2 x 28 MiB, allocated by hbt_mlp_create): calls on ONE handle
+ * must therefore not overlap, on any streams; different handles are
+ * independent.  Results are reproducible for a given n and position of the
+ * row; the paths (per layer with K split over workgroups or waves in several
+ * ways by row count, fused) sum in different orders and agree to fp32
  * rounding.
  */
 int hbt_mlp_forward(hbt_mlp *mlp, const double *raw_features, int64_t n, float *out,

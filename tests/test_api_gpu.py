@@ -425,7 +425,28 @@ def test_local_device_description_and_measured_ceilings():
     from habitat_amd import DeviceProperties
     dev = DeviceProperties(name="local", **props)        # the keys are DeviceProperties' own
     assert dev.num_sms == props["num_sms"]
-    m = device_info.measure(iters=2000, copy_bytes=1 << 28)
+    m = device_info.measure(iters=20000, copy_bytes=1 << 30)
     # an MI355X: several TB/s of copy bandwidth, tens of TFLOP/s of fp32
     assert m["copy_gbps"] > 500 and m["fp32_fma_gflops"] > 5000 and m["fp32_mfma_gflops"] > 20000
     assert m["fp32_mfma_gflops"] > m["fp32_fma_gflops"]
+    # The three figures derived from the reported clocks (the table's
+    # mem_bandwidth_gb, base_clock_mhz, peak_gflops_per_second), held against
+    # what the box measures and what is published for the MI355X: the bandwidth
+    # lies between the measured copy rate and the published 8 TB/s (8192 GB/s
+    # by the clocks), the clock in 2.0-2.5 GHz, the vector fp32 peak within 15 %
+    # above the measured FMA rate and at half the published 157.3 TFLOP/s,
+    # which counts packed fp32 or the matrix cores.
+    assert m["copy_gbps"] < props["mem_bandwidth_gb"] <= 8000 * 1.03
+    assert 2000 <= props["base_clock_mhz"] <= 2500
+    assert m["fp32_fma_gflops"] <= props["peak_gflops_per_second"] <= 1.15 * m["fp32_fma_gflops"]
+    assert props["peak_gflops_per_second"] == pytest.approx(157300 / 2, rel=0.02)
+    assert m["fp32_mfma_gflops"] == pytest.approx(157300, rel=0.05)
+    # the reading as a compute-unit description: the GPU of the table's MI355X_cdna row
+    from habitat_amd.analysis.wave_scaling.cdna import native_description
+    native = native_description(dev).as_dict()
+    table = Device.MI355X_cdna.as_dict()
+    for key in ("compute_major", "compute_minor", "max_threads_per_block",
+                "max_threads_per_multiprocessor", "regs_per_multiprocessor", "warp_size",
+                "shared_mem_per_block", "shared_mem_per_multiprocessor", "num_sms",
+                "base_clock_mhz"):
+        assert native[key] == table[key], key
