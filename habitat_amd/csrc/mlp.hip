@@ -570,7 +570,20 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
 // k-group (km_index); bias and ReLU are applied on the way out.
 // Measured per forward at 4096 rows with KS = 1: a wave owning 2 x 2 tiles 526
 // us, 1 x 2 tiles 514, one tile 501 (8 ring slots: 503); workgroups numbered
-// m-tile first instead of n-tile first: no difference.
+// m-tile first instead of n-tile first: no difference.  Workgroups of 8 or 16
+// waves with K in as many parts (a tile per workgroup, everything summed in
+// LDS) took 57-59 us at 21 to 128 rows, where two workgroups per tile with their
+// K-partials through memory take 49-58: a tile is 3.4 us of ONE compute unit's
+// matrix cores, so few rows want each tile spread over several compute units.
+// fc2 folded into the last hidden layer (every wave leaves its tile's share of
+// the dot product in memory, the wave that completes an m-tile's 32 shares adds
+// them in order; no launch for fc2, no activations written) gained nothing: 512
+// rows 102 us against 99, 4096 rows 511 against 506, 160 rows 60 against 62 -
+// the fc2 launch costs what the count-and-add tail costs (with __threadfence
+// around the count 4096 rows took 591 us: the fences' cache invalidations cost
+// the waves still in their K loop their weights).  A separate fc1 kernel (a
+// workgroup per m-tile standardising the rows once for all n-tiles) was slower
+// below 1024 rows and within 1 % above.
 template <int KS, int SLOTS>
 __global__ __launch_bounds__(256) void mlp_layer_tile_kernel(const LayerArgs a) {
   static_assert(KS == 1 || KS == 2 || KS == 4, "four waves per workgroup");
