@@ -318,6 +318,11 @@ constexpr int kLayerMaxRows = 7168;
 // Measured per forward at 32 / 64 / 128 / 256 rows: 49 52 58 82 us against 57 57
 // 59 65 without; four K-partials were no faster than two.
 constexpr int kHalfKMaxTiles = 4;
+// Input features up to which fc1 of a batch stored by k-group is computed with
+// plain FMAs (mlp_first_fma_kernel); the reference's networks have 8 to 12.
+constexpr int kFirstFmaMaxIn = 16;
+constexpr int kFirstFmaSlices = 8;     // workgroups per m-tile (gridDim.y)
+constexpr int kFirstFmaMinTiles = 64;  // m-tiles from which that kernel is used (2048 rows)
 constexpr size_t kScratchFloats = (size_t)kLayerMaxRows * kWidth;  // each of two buffers
 static_assert((size_t)kSplit * kRows * kWidth <= kScratchFloats, "the K-partials fit the scratch");
 
@@ -337,6 +342,7 @@ struct LayerArgs {
   int64_t n;
   int32_t m_pad;           // rows rounded up to 32
   float* p_out;            // m_pad x kWidth activations (FINAL), else `splits` blocks of partials
+  const float* w_first_t;  // fc1.weight transposed, [kFirstFmaMaxIn][kWidth] (mlp_first_fma_kernel)
 };
 
 // Outside the split-K shape activations are stored by k-group (KM below): element
@@ -672,6 +678,60 @@ __global__ __launch_bounds__(256) void mlp_layer_tile_kernel(const LayerArgs a) 
   }
 }
 
+// fc1 for large batches stored by k-group, with at most kFirstFmaMaxIn input
+// features: K is a dozen, so the layer is its 4 KiB-per-row write and little
+// else, and plain FMAs from LDS do it without the matrix cores.  A workgroup
+// takes one m-tile and an eighth of the outputs: it standardises the m-tile's
+// raw fp64 rows (the 4-wave MFMA kernel does that once per n-tile, 32 times per
+// row, this one 8 times), stages its slice of the transposed weights in LDS,
+// and each lane (row m, half h) then produces four consecutive outputs per
+// k-group of the next layer, 1 KiB of contiguous memory per wave and store.
+// Sum order: bias, then k ascending.  Measured against the MFMA kernel: 4096
+// rows 8.4 against 14.1 us, 1536 rows 7.2 against 6.8, 512 rows 5.3 against 4.5
+// (hence kFirstFmaMinTiles); with 2 / 16 / 32 slices instead of 8, 4096 rows take
+// 19.4 / 10.0 / 13.6 us.
+__global__ __launch_bounds__(256) void mlp_first_fma_kernel(const LayerArgs a) {
+  __shared__ float xs[kRows][kFirstFmaMaxIn + 1];
+  __shared__ __attribute__((aligned(16))) float wl[kFirstFmaMaxIn * (kWidth / kFirstFmaSlices)];  // [k][n of the slice]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 31, h = lane >> 5;
+  const int m_tile = blockIdx.x;
+  constexpr int slice_n = kWidth / kFirstFmaSlices;  // outputs of this workgroup
+  const int n_base = (int)blockIdx.y * slice_n;
+  for (int idx = tid; idx < kRows * kFirstFmaMaxIn; idx += 256) {
+    const int r = idx / kFirstFmaMaxIn, k = idx - r * kFirstFmaMaxIn;
+    const int64_t row = (int64_t)m_tile * kRows + r;
+    float v = 0.f;
+    if (k < a.in_features && row < a.n)
+      v = (float)((a.raw[row * a.in_features + k] - a.mu[k]) / a.sigma[k]);
+    xs[r][k] = v;
+  }
+  for (int idx = tid; idx < a.in_features * (slice_n / 4); idx += 256) {
+    const int k = idx / (slice_n / 4), c = idx - k * (slice_n / 4);
+    *reinterpret_cast<f32x4*>(wl + k * slice_n + 4 * c) =
+        *reinterpret_cast<const f32x4*>(a.w_first_t + (size_t)k * kWidth + n_base + 4 * c);
+  }
+  __syncthreads();
+  float x[kFirstFmaMaxIn];
+#pragma unroll
+  for (int k = 0; k < kFirstFmaMaxIn; ++k) x[k] = xs[m][k];
+  for (int g = wave; g < slice_n / 8; g += 4) {
+    const int local = 8 * g + 4 * h, n0 = n_base + local;
+    f32x4 o = *reinterpret_cast<const f32x4*>(a.bias_out + n0);
+#pragma unroll
+    for (int k = 0; k < kFirstFmaMaxIn; ++k)
+      if (k < a.in_features) {
+        const f32x4 w = *reinterpret_cast<const f32x4*>(wl + k * slice_n + local);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = fmaf(x[k], w[e], o[e]);
+      }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = relu(o[e]);
+    *reinterpret_cast<f32x4*>(a.p_out + km_index(m_tile, n0 >> 3, m, 4 * h)) = o;
+  }
+}
+
 struct LastArgs {
   const float* p_in;     // m_pad x kWidth activations, or S_IN such blocks of K-partials
   const float* bias_in;  // [kWidth], bias of the last hidden layer (with partials)
@@ -787,6 +847,7 @@ struct hbt_mlp {
   const float* w_stream;
   const float* bias;
   const float* w_last;
+  const float* w_first_t;  // fc1.weight transposed [kFirstFmaMaxIn][width]; null above that many inputs
   float b_last;
   float* scratch[2];   // per-layer path: two buffers of kScratchFloats activations or partials
 };
@@ -895,6 +956,7 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
   l.in_features = mlp->in_features;
   l.n = n;
   l.m_pad = m_tiles * kRows;
+  l.w_first_t = mlp->w_first_t;
   bool partials = false;
   const float* p_in = nullptr;
   const int tile_ks = tile_k_parts(m_tiles);
@@ -910,7 +972,10 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
     if (layer == 0 && split_k)
       hipLaunchKernelGGL((mlp_layer_kernel<true, 0, true, 4, false, 0>), grid, dim3(256), 0,
                          stream, l);
-    else if (layer == 0)
+    else if (layer == 0 && mlp->w_first_t != nullptr && m_tiles >= kFirstFmaMinTiles) {
+      hipLaunchKernelGGL(mlp_first_fma_kernel, dim3((unsigned)m_tiles, kFirstFmaSlices), dim3(256), 0,
+                         stream, l);
+    } else if (layer == 0)
       hipLaunchKernelGGL((mlp_layer_kernel<true, 0, true, 4, false, 0, 1, true>), grid, dim3(256),
                          0, stream, l);
     else if (ks == 2 && !partials)
@@ -1027,6 +1092,9 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
   const size_t off_stream = off; off = align_up(off + sizeof(float) * n_stream, 256);
   const size_t off_bias = off; off = align_up(off + sizeof(float) * n_bias, 256);
   const size_t off_last = off; off = align_up(off + sizeof(float) * kWidth, 256);
+  const bool first_fma = in_features <= kFirstFmaMaxIn;
+  const size_t off_first_t = off;
+  if (first_fma) off = align_up(off + sizeof(float) * kFirstFmaMaxIn * kWidth, 256);
   const size_t image = off;  // what is copied from the host; scratch follows
   const size_t scratch_bytes = sizeof(float) * kScratchFloats;
   const size_t off_scratch0 = off; off = align_up(off + scratch_bytes, 256);
@@ -1051,6 +1119,11 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
     std::memcpy(host.data() + off_bias + sizeof(float) * (size_t)l * kWidth, b[l],
                 sizeof(float) * kWidth);
   std::memcpy(host.data() + off_last, W[hidden_layers + 1], sizeof(float) * kWidth);
+  if (first_fma) {
+    float* t = reinterpret_cast<float*>(host.data() + off_first_t);  // zero beyond in_features
+    for (int n = 0; n < kWidth; ++n)
+      for (int k = 0; k < in_features; ++k) t[(size_t)k * kWidth + n] = W[0][(size_t)n * in_features + k];
+  }
 
   void* blob = nullptr;
   if (hipMalloc(&blob, total) != hipSuccess) {
@@ -1092,6 +1165,7 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
   m->w_stream = reinterpret_cast<const float*>(base + off_stream);
   m->bias = reinterpret_cast<const float*>(base + off_bias);
   m->w_last = reinterpret_cast<const float*>(base + off_last);
+  m->w_first_t = first_fma ? reinterpret_cast<const float*>(base + off_first_t) : nullptr;
   m->b_last = b[hidden_layers + 1][0];
   m->scratch[0] = reinterpret_cast<float*>(base + off_scratch0);
   m->scratch[1] = reinterpret_cast<float*>(base + off_scratch1);
