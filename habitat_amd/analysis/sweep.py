@@ -161,18 +161,41 @@ class SweepCall:
                                     [P.occupancy_device(dests[i], plan.mode) for i in idxs])
                 at = None if whole else torch.tensor(idxs, device=plan.gpu)
                 self.groups.append((rec, table, at))
-        self.dev_feats = None
         self.streams = [torch.cuda.Stream(plan.gpu) for _ in plan.special]   # default priority
+        # The MLP input rows of every kind, (destinations + origin) x distinct
+        # operation rows: they depend on the plan and the destinations only, so
+        # they are laid out here, once, and `launch` just runs the networks.
+        self.rows = {}
         if plan.special:
-            self.dev_feats = torch.tensor(
+            D = len(dests)
+            dev_feats = torch.tensor(
                 np.asarray([feats_of(d) for d in dests] + [feats_of(plan.origin)], np.float64),
                 device=plan.gpu)                                                      # [D + 1, 4]
+            for kind, (idxs, pred, op_feats, ms, op_row) in plan.special.items():
+                U = op_feats.shape[0]
+                self.rows[kind] = torch.cat(
+                    [op_feats.unsqueeze(0).expand(D + 1, U, -1),
+                     dev_feats.unsqueeze(1).expand(D + 1, U, 4)], dim=2).reshape((D + 1) * U, -1)
 
     def launch(self):
         plan, D = self.plan, len(self.dests)
         res = TraceSweep()
         res.pass_overhead_ns = plan.pass_overhead_ns
         res.pass_owner = plan.pass_owner
+        # One MLP forward per kind, each on a stream of its own and enqueued
+        # first: a kind with few operations fills a fraction of the GPU, so the
+        # kinds run side by side, and the wave-scaling sums of the main stream
+        # run beside them instead of in front of them.
+        main = torch.cuda.current_stream(plan.gpu)
+        preds = {}
+        for (kind, (idxs, pred, op_feats, ms, op_row)), side in zip(plan.special.items(),
+                                                                    self.streams):
+            U = op_feats.shape[0]
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                y = pred.predict_batch(self.rows[kind]).view(D + 1, U)
+            y.record_stream(main)
+            preds[kind] = y
         total = torch.full((D,), plan.const_ms, dtype=torch.float64, device=plan.gpu)
         if self.groups:
             if len(self.groups) == 1 and self.groups[0][2] is None:
@@ -192,21 +215,6 @@ class SweepCall:
         else:
             res.pass_kernel_ns = torch.zeros((D, plan.n_seg), dtype=torch.float64, device=plan.gpu)
             res.bad_records = torch.zeros((D,), dtype=torch.int32, device=plan.gpu)
-        # One MLP launch per kind, each on a stream of its own: a kind with few
-        # operations fills a fraction of the GPU, so the kinds run side by side.
-        main = torch.cuda.current_stream(plan.gpu)
-        preds = {}
-        for (kind, (idxs, pred, op_feats, ms, op_row)), side in zip(plan.special.items(),
-                                                                    self.streams):
-            U = op_feats.shape[0]
-            side.wait_stream(main)
-            with torch.cuda.stream(side):
-                rows = torch.cat([op_feats.unsqueeze(0).expand(D + 1, U, -1),
-                                  self.dev_feats.unsqueeze(1).expand(D + 1, U, 4)], dim=2)
-                y = pred.predict_batch(rows.reshape((D + 1) * U, -1)).view(D + 1, U)
-            rows.record_stream(main)
-            y.record_stream(main)
-            preds[kind] = y
         for side in self.streams:
             main.wait_stream(side)
         res.clamped_ops = torch.zeros((D,), dtype=torch.int32, device=plan.gpu)
