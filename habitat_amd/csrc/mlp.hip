@@ -576,7 +576,10 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
 // k-group (km_index); bias and ReLU are applied on the way out.
 // Measured per forward at 4096 rows with KS = 1: a wave owning 2 x 2 tiles 526
 // us, 1 x 2 tiles 514, one tile 501 (8 ring slots: 503); workgroups numbered
-// m-tile first instead of n-tile first: no difference.  Workgroups of 8 or 16
+// m-tile first instead of n-tile first: no difference; two accumulators taking
+// turns (no MFMA waits for the one before it): no difference up to 5120 rows, and
+// above that the 16 registers more cost residency (5911 rows 936 us against 730).
+// Workgroups of 8 or 16
 // waves with K in as many parts (a tile per workgroup, everything summed in
 // LDS) took 57-59 us at 21 to 128 rows, where two workgroups per tile with their
 // K-partials through memory take 49-58: a tile is 3.4 us of ONE compute unit's
