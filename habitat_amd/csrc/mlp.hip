@@ -280,27 +280,27 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
 }
 
 // ---------------------------------------------------------------------------
-// Up to a few thousand rows (one prediction, the operations of one trace, a
-// trace for some devices): one launch per layer.
+// Up to kLayerMaxRows rows (one prediction, the operations of one trace, a trace
+// for some devices): one launch per layer.
 //
 // The fused kernel gives each workgroup 32 rows and the whole network, so a
 // batch of up to 32 rows runs on ONE compute unit, which has to pull all
 // 33.6 MB of weights through by itself (about 1 ms), and any batch below 8192
 // rows leaves compute units idle for that long.  Here a layer is spread over
-// the chip instead: a workgroup takes one or two n-tiles x one m-tile, its
-// waves split K, each multiplies its k-groups straight from global memory (no
-// loop, no LDS staging) and the waves add their 32 x 32 accumulators through
-// LDS.
+// the chip instead, in one of three shapes:
 //
-//   For a few rows (up to kSplitMaxRows) K is split kSplit ways over
-//   workgroups as well (four waves, 4 k-groups each: 256 workgroups) and the
-//   K-partials are written as they are, [split][row][n]; they are summed,
-//   biased and rectified by whoever reads them: the next layer's activation
-//   load, or the final dot product.
-//   Otherwise eight waves cover all of K (16 k-groups each), the workgroup
-//   applies bias and ReLU and writes activations, stored by k-group (see
-//   km_index).  Up to kHalfKMaxTiles m-tiles K is split over two such
-//   workgroups, whose K-partials are stored by k-group too.
+//   For a few rows (up to kSplitMaxRows) mlp_layer_kernel with four waves: a
+//   workgroup takes one n-tile x one m-tile and an eighth of K (kSplit: 256
+//   workgroups per layer), its waves split that eighth, each multiplies its
+//   k-groups straight from global memory (no loop, no LDS staging), the waves
+//   add their 32 x 32 accumulators through LDS, and the K-partials are written
+//   as they are, [split][row][n]; they are summed, biased and rectified by
+//   whoever reads them: the next layer's activation load, or the final dot
+//   product.
+//   Up to kHalfKMaxTiles m-tiles (128 rows) the same kernel with eight waves
+//   and K over two workgroups, whose K-partials are stored by k-group (see
+//   km_index), like all activations from here on.
+//   Above that mlp_layer_tile_kernel: a wave per output tile, see there.
 //
 // The order of every sum is fixed, so results are reproducible.  Same packed
 // weights, same MFMA instruction, same fragment layout as above.
@@ -323,7 +323,7 @@ constexpr int kHalfKMaxTiles = 4;
 constexpr int kFirstFmaMaxIn = 16;
 constexpr int kFirstFmaSlices = 8;     // workgroups per m-tile (gridDim.y)
 constexpr int kFirstFmaMinTiles = 64;  // m-tiles from which that kernel is used (2048 rows)
-constexpr size_t kScratchFloats = (size_t)kLayerMaxRows * kWidth;  // each of two buffers
+constexpr size_t kScratchFloats = (size_t)kLayerMaxRows * kWidth;  // each of two buffers (28 MiB)
 static_assert((size_t)kSplit * kRows * kWidth <= kScratchFloats, "the K-partials fit the scratch");
 
 struct LayerArgs {
@@ -385,16 +385,18 @@ struct LayerFrag {
 //     other).
 //   KM: activations (read, unless FIRST, and written) are stored by k-group.
 //   S_OUT: K-partials this launch writes (a.splits; 1 with FINAL).
-// Measured for the whole-K shape with KM, us per forward at 256 / 512 / 768 /
-// 1024 / 1536 / 2048 / 4096 rows, as (DEPTH, NT):
+// The instantiations in use: fc1 (FIRST, FINAL, 4 waves) with row-major or
+// k-group output; hidden layers with kSplit K-partials in and out (4 waves,
+// rows masked); hidden layers with two K-partials in and out (8 waves, DEPTH 2,
+// KM).  Until mlp_layer_tile_kernel took over above 128 rows, the eight-wave
+// whole-K shape (FINAL, S_IN 0) ran there; measured for it with KM, us per
+// forward at 256 / 512 / 768 / 1024 / 1536 / 2048 / 4096 rows, as (DEPTH, NT):
 //   (0,1)  67 103 128 161 251 318 588     (0,2) 105 110 160 162 230 298 560
 //   (2,1)  67 103 130 160 274 319 596     (2,2)  95 100 154 154 280 291 605
 //   (4,1)  66 104 130 190 231 325 598     (0,4) 168 172 170 171 310 320 613
 //   (16,1) 71 116 154 194 277 360 693     (2,4) 157 161 158 159 287 299 567
-// so below 1024 rows a workgroup takes one n-tile with two groups in flight,
-// from there on two n-tiles and the compiler's placement.  (With row-major
-// activations, where a fragment touches 32 cache lines for 32 bytes each: 256
-// rows 74 us, 512 123, 1024 176 with four n-tiles, 4096 637.)
+// (with row-major activations, where a fragment touches 32 cache lines for 32
+// bytes each: 256 rows 74 us, 512 123, 1024 176 with four n-tiles, 4096 637).
 template <bool FIRST, int S_IN, bool FINAL, int WAVES, bool PADDED_ROWS, int DEPTH, int NT = 1,
           bool KM = false, int S_OUT = (FINAL ? 1 : kSplit)>
 __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a) {
