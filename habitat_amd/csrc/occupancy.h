@@ -392,7 +392,7 @@ HBT_HD int32_t occupancy_core(const OccDevice& d, int32_t block, int32_t smem_to
   {
     // C division truncates toward zero: (total + 255) / 256 * 256.
     const int64_t t255 = (int64_t)smem_total + 255;
-    const int64_t alloc = (t255 >= 0 ? (t255 >> 8) : -((-t255) >> 8)) << 8;
+    const int64_t alloc = (t255 >= 0 ? (t255 >> 8) : -((-t255) >> 8)) * 256;
     if (alloc < 0 || alloc > d.smem_per_block) {
       lim_smem = 0;
     } else if (alloc == 0) {
