@@ -466,8 +466,9 @@ def main():
         dt = time.perf_counter() - t0
         return {"scalar_strategy_us_per_kernel": dt / m * 1e6, "kernels": m, "raised": skipped,
                 "what": "unified_wave_scaling(kernel, origin, dest, manager), the reference's "
-                        "strategy signature (predictor.py:116-124): per call one 64-byte upload, "
-                        "one launch, one 24-byte read-back and a wait"}
+                        "strategy signature (predictor.py:116-124): per call one "
+                        "hbt_wave_scale_one, i.e. one launch on a pinned device-visible record "
+                        "and a wait"}
 
     attempt("scalar_strategy", scalar_section)
 

@@ -9,7 +9,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libhabitat_mi.so")
 
-ABI_VERSION = 101   # HBT_VERSION of include/habitat_mi.h this binding was written for
+ABI_VERSION = 102   # HBT_VERSION of include/habitat_mi.h this binding was written for
 
 MLP_STATIC_MAX_ROWS = 1024   # HBT_MLP_STATIC_MAX_ROWS
 
@@ -28,6 +28,17 @@ class DeviceSpec(C.Structure):
         ("smem_per_block_optin", C.c_int64),
         ("mem_bandwidth_gb", C.c_double), ("base_clock_mhz", C.c_double),
         ("peak_gflops", C.c_double),
+    ]
+
+
+class KernelRecord(C.Structure):
+    """hbt_kernel_record."""
+    _fields_ = [
+        ("num_blocks", C.c_int32), ("block_size", C.c_int32), ("dynamic_smem", C.c_int32),
+        ("static_smem", C.c_int32), ("regs", C.c_int32), ("dest_regs", C.c_int32),
+        ("has_metrics", C.c_int32), ("reserved", C.c_int32),
+        ("run_time_ns", C.c_double), ("flop_sp_efficiency", C.c_double),
+        ("dram_read_bytes", C.c_double), ("dram_write_bytes", C.c_double),
     ]
 
 
@@ -52,6 +63,10 @@ _SIGNATURES = {
                                                    _P]),
     "hbt_wave_scale": (C.c_int, [C.POINTER(DeviceSpec), C.POINTER(DeviceSpec), C.c_int32,
                                  C.c_int64] + [_P] * 17 + [_P]),
+    "hbt_wave_scale_one": (C.c_int, [C.POINTER(DeviceSpec), C.POINTER(DeviceSpec),
+                                     C.POINTER(KernelRecord), C.POINTER(C.c_double),
+                                     C.POINTER(C.c_int32), C.POINTER(C.c_int32),
+                                     C.POINTER(C.c_uint8), _P]),
     "hbt_device_table_create": (_P, [C.POINTER(DeviceSpec), C.POINTER(DeviceSpec), C.c_int32,
                                      C.POINTER(C.c_int)]),
     "hbt_device_table_size": (C.c_int32, [_P]),

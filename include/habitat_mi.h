@@ -6,10 +6,11 @@
  * parameter says "host", every array pointer is DEVICE memory owned by the
  * caller; work is enqueued on the given HIP stream (NULL = the default stream)
  * and the call returns without synchronising.  Functions return 0 or a
- * negative HBT_E* code; hbt_strerror() names it.  There is no global state and
- * no CPU fallback: without a GPU the compute entry points return HBT_EHIP.
- * Only the two *_create calls allocate device memory (and the calibration
- * calls at the end, which say so).
+ * negative HBT_E* code; hbt_strerror() names it.  There is no CPU fallback:
+ * without a GPU the compute entry points return HBT_EHIP.  Only the two
+ * *_create calls allocate device memory (and the calibration calls at the
+ * end, which say so); the library's only state outside its handles is what
+ * hbt_wave_scale_one and hbt_mlp_forward_static say they keep per GPU.
  *
  * Each entry point cites the reference interface it stands in for
  * (paths relative to the reference tree).
@@ -24,7 +25,7 @@
 extern "C" {
 #endif
 
-#define HBT_VERSION 101 /* 0.1.1 */
+#define HBT_VERSION 102 /* 0.1.2 */
 
 enum {
   HBT_OK = 0,
@@ -158,6 +159,32 @@ int hbt_wave_scale(const hbt_device_spec *origin, const hbt_device_spec *dests, 
                    double *out_time_ns, int32_t *out_occ_origin, int32_t *out_occ_dest,
                    int32_t *out_wave_origin, int32_t *out_wave_dest, uint8_t *out_status,
                    void *hip_stream);
+
+/*
+ * One kernel record, one destination, start to finish: the reference's strategy
+ * call  strategy(kernel, origin_device, dest_device, metadata_manager)
+ * (analysis/predictor.py:116-124 invoking wave_scaling/unified.py:8-35) as one C
+ * call.  `record` and the out pointers are HOST memory.  The record goes through
+ * a pinned, device-visible staging block of the library (128 bytes per GPU,
+ * allocated on the first call there and kept), the same kernel as
+ * hbt_wave_scale runs on it on `hip_stream`, and the call waits for the stream
+ * before it returns: some 15 us, all of it launch and wait (21 us per kernel
+ * through the Python strategy that wraps it).  dest_regs < 0 =
+ * no register-table entry; has_metrics == 0 selects the no-metrics strategy.
+ * *out_status is one of HBT_ST_*; the time is NaN unless it is HBT_ST_OK.
+ * out_occ_origin and out_occ_dest are nullable.  Calls on one GPU are
+ * serialised inside the library.  Callers with many kernels should hand them
+ * over together (hbt_wave_scale).
+ */
+typedef struct hbt_kernel_record {
+  int32_t num_blocks, block_size, dynamic_smem, static_smem, regs, dest_regs;
+  int32_t has_metrics, reserved;
+  double run_time_ns, flop_sp_efficiency, dram_read_bytes, dram_write_bytes;
+} hbt_kernel_record;
+int hbt_wave_scale_one(const hbt_device_spec *origin, const hbt_device_spec *dest,
+                       const hbt_kernel_record *record, double *out_time_ns,
+                       int32_t *out_occ_origin, int32_t *out_occ_dest, uint8_t *out_status,
+                       void *hip_stream);
 
 /*
  * A set of destination devices resident on the GPU, for predicting one trace

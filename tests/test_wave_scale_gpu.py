@@ -98,6 +98,75 @@ def test_hand_worked_known_answers_through_the_batch_kernel(kat):
                 assert g[i] == pytest.approx(r["gamma"], rel=1e-12), r
 
 
+def test_one_record_entry_point_through_the_c_abi(kat):
+    """hbt_wave_scale_one (a host record in, time / occupancies / status out,
+    synchronous) against the hand-worked known answers, against the batch entry
+    point bit for bit on ordinary and adversarial records, and its argument
+    checks."""
+    import ctypes
+    from habitat_amd import _lib
+    L = _lib.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def one(origin, dest, rec_fields):
+        rec = _lib.KernelRecord(**rec_fields)
+        t, st = ctypes.c_double(-1.0), ctypes.c_uint8(99)
+        oo, od = ctypes.c_int32(-7), ctypes.c_int32(-7)
+        rc = L.hbt_wave_scale_one(ctypes.byref(origin.spec), ctypes.byref(dest.spec),
+                                  ctypes.byref(rec), ctypes.byref(t), ctypes.byref(oo),
+                                  ctypes.byref(od), ctypes.byref(st), stream)
+        assert rc == 0
+        return t.value, oo.value, od.value, st.value
+
+    base = kat["scaling_record"]
+    for row in kat["scaling"]:
+        over = row.get("record", {})
+        fields = dict(num_blocks=row["num_blocks"], block_size=base["block_size"],
+                      dynamic_smem=base["dynamic_smem"], static_smem=base["static_smem"],
+                      regs=base["regs_per_thread"], dest_regs=row.get("dest_regs", -1),
+                      has_metrics=int(row.get("has_metrics", True)),
+                      run_time_ns=float(base["run_time_ns"]),
+                      flop_sp_efficiency=over.get("flop_sp_efficiency", base["flop_sp_efficiency"]),
+                      dram_read_bytes=base["dram_read_bytes"],
+                      dram_write_bytes=base["dram_write_bytes"])
+        t, oo, od, st = one(getattr(Device, row["origin"]), getattr(Device, row["dest"]), fields)
+        assert st == 0 and t == pytest.approx(row["time_ns"], rel=TIME_RTOL), row
+        if "occ_origin" in row:
+            assert oo == row["occ_origin"]
+        if "occ_dest" in row:
+            assert od == row["occ_dest"]
+    # the same kernel as the batch call: identical bits, record by record
+    for rec in (synthetic.kernel_records(300, Device.V100, seed=31, metrics_fraction=0.7)[0],
+                adversarial_records(300, 5)):
+        out = wave_scale(KernelRecords.from_numpy(rec), Device.V100, [Device.T4])
+        bt, bs = out.time_ns[0].cpu().numpy(), out.status[0].cpu().numpy()
+        bo, bd = out.occ_origin.cpu().numpy(), out.occ_dest[0].cpu().numpy()
+        for i in range(300):
+            fields = dict(num_blocks=int(rec["num_blocks"][i]), block_size=int(rec["block_size"][i]),
+                          dynamic_smem=int(rec["dynamic_smem"][i]),
+                          static_smem=int(rec["static_smem"][i]), regs=int(rec["regs_per_thread"][i]),
+                          dest_regs=int(rec["dest_regs"][i]) if "dest_regs" in rec else -1,
+                          has_metrics=int(rec["has_metrics"][i]) if "has_metrics" in rec else 1,
+                          run_time_ns=float(rec["run_time_ns"][i]),
+                          flop_sp_efficiency=float(rec["flop_sp_efficiency"][i]),
+                          dram_read_bytes=float(rec["dram_read_bytes"][i]),
+                          dram_write_bytes=float(rec["dram_write_bytes"][i]))
+            t, oo, od, st = one(Device.V100, Device.T4, fields)
+            assert (st, oo, od) == (bs[i], bo[i], bd[i]), i
+            assert t == bt[i] or (math.isnan(t) and math.isnan(bt[i])), i
+    # argument checks
+    rec = _lib.KernelRecord()
+    t, st = ctypes.c_double(0), ctypes.c_uint8(0)
+    v100 = ctypes.byref(Device.V100.spec)
+    assert L.hbt_wave_scale_one(v100, v100, None, ctypes.byref(t), None, None, ctypes.byref(st),
+                                stream) == _lib.HBT_EINVAL
+    assert L.hbt_wave_scale_one(v100, v100, ctypes.byref(rec), None, None, None, ctypes.byref(st),
+                                stream) == _lib.HBT_EINVAL
+    bad = DeviceProperties(name="z", **dict(Device.V100.as_dict(), base_clock_mhz=0))
+    assert L.hbt_wave_scale_one(v100, ctypes.byref(bad.spec), ctypes.byref(rec), ctypes.byref(t),
+                                None, None, ctypes.byref(st), stream) == _lib.HBT_ESPEC
+
+
 def test_identity_and_round_trip_properties():
     rec, _ = synthetic.kernel_records(200_000, Device.V100, seed=3, metrics_fraction=0.5)
     kr = KernelRecords.from_numpy(rec)
