@@ -105,6 +105,38 @@ def test_scalar_strategies_raise_what_the_reference_raises():
                                      mm).run_time_ns == 1000000
 
 
+def test_scalar_strategy_from_several_threads():
+    """The one-kernel call shares a staging block per GPU inside the library
+    and serialises its callers: four threads scaling different kernels at once
+    each get their own kernel's answer."""
+    import threading
+    mm = NullMetadataManager()
+    origin, dest = Device.V100, Device.T4
+    kernels = [make_kernel(origin, num_blocks=64 + 997 * i, t_ns=1_000_000 + 12_345 * i,
+                           metrics=(10.0 + i, 1e8, 2e8) if i % 3 else None) for i in range(64)]
+    want = [unified_wave_scaling(k, origin, dest, mm).run_time_ns for k in kernels]
+    assert len(set(want)) > 32
+    got = [None] * len(kernels)
+    errors = []
+
+    def work(start):
+        try:
+            torch.cuda.set_device(0)
+            for _ in range(5):
+                for i in range(start, len(kernels), 4):
+                    got[i] = unified_wave_scaling(kernels[i], origin, dest, mm).run_time_ns
+        except Exception as exc:       # noqa: BLE001 - reported below
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert got == want
+
+
 def test_scalar_strategy_uses_the_register_table():
     k = make_kernel(Device.V100, num_blocks=400, name="gemm")
     rec = as_record(k, (50.0, 1e8, 1e8))
