@@ -42,6 +42,13 @@ constexpr int kRecPerThread = kVectorRecords;
 // thread: 64 threads 11.7 us, 128 11.9, 256 12.5, 512 13.5, and 512 was the only
 // size that ran faster, 12.3 us, for the first milliseconds after idle.)
 constexpr int kBlock = 128;
+// Tried and dropped: a smaller grid whose waves walk over the batch in strides of
+// the whole grid and issue the loads of their next 64 records before computing
+// on the ones they hold (74 VGPRs, 6 waves per SIMD).  1 M records: 11.8 us with
+// 5209 workgroups (1.5 turns per wave), 12.5-13.7 with 2605-3907, 15.1 with 1563,
+// against 11.3; 64 M records 890-960 us against 696.  Fresh short waves taking
+// consecutive chunks keep the chip on one contiguous window of every column;
+// waves that come back for chunks a whole grid further on do not.
 
 // N consecutive elements as one register group (a scalar when N is 1).
 template <class T, int N>
