@@ -464,11 +464,35 @@ def main():
             except ZeroDivisionError:      # destination occupancy 0: the reference raises too
                 skipped += 1
         dt = time.perf_counter() - t0
+        # the same loop shape with the deferred strategy: note every kernel, then
+        # read every time (the first read hands the whole set to the GPU)
+        from habitat_amd.analysis.wave_scaling.deferred import deferred_unified_wave_scaling
+
+        def deferred_pass(ks):
+            t0 = time.perf_counter()
+            preds = [deferred_unified_wave_scaling(k, origin, dest, mm) for k in ks]
+            total, raised = 0.0, 0
+            for p in preds:
+                try:
+                    total += p.run_time_ns
+                except ZeroDivisionError:
+                    raised += 1
+            return (time.perf_counter() - t0) / len(ks) * 1e6, raised
+
+        first_us, d_raised = deferred_pass(kernels)       # packs every kernel's record
+        again_us = min(deferred_pass(kernels)[0] for _ in range(5))
+        trace_sized_us = min(deferred_pass(kernels[:900])[0] for _ in range(5))
         return {"scalar_strategy_us_per_kernel": dt / m * 1e6, "kernels": m, "raised": skipped,
+                "deferred_us_per_kernel": again_us,
+                "deferred_us_per_kernel_900_kernels": trace_sized_us,
+                "deferred_first_pass_us_per_kernel": first_us, "deferred_raised": d_raised,
                 "what": "unified_wave_scaling(kernel, origin, dest, manager), the reference's "
                         "strategy signature (predictor.py:116-124): per call one "
                         "hbt_wave_scale_one, i.e. one launch on a pinned device-visible record "
-                        "and a wait"}
+                        "and a wait.  deferred_*: deferred_unified_wave_scaling in the same "
+                        "loop, times read afterwards as run_time.py:50-58 does: one "
+                        "hbt_wave_scale_host_records call for the whole set; first pass = "
+                        "including the one-time packing of each kernel object's record"}
 
     attempt("scalar_strategy", scalar_section)
 

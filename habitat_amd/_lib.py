@@ -9,7 +9,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libhabitat_mi.so")
 
-ABI_VERSION = 102   # HBT_VERSION of include/habitat_mi.h this binding was written for
+ABI_VERSION = 103   # HBT_VERSION of include/habitat_mi.h this binding was written for
 
 MLP_STATIC_MAX_ROWS = 1024   # HBT_MLP_STATIC_MAX_ROWS
 
@@ -67,6 +67,8 @@ _SIGNATURES = {
                                      C.POINTER(KernelRecord), C.POINTER(C.c_double),
                                      C.POINTER(C.c_int32), C.POINTER(C.c_int32),
                                      C.POINTER(C.c_uint8), _P]),
+    "hbt_wave_scale_host_records": (C.c_int, [C.POINTER(DeviceSpec), C.POINTER(DeviceSpec),
+                                              C.c_int64, _P, _P, _P, _P, _P, _P]),
     "hbt_device_table_create": (_P, [C.POINTER(DeviceSpec), C.POINTER(DeviceSpec), C.c_int32,
                                      C.POINTER(C.c_int)]),
     "hbt_device_table_size": (C.c_int32, [_P]),

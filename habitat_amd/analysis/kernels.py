@@ -5,6 +5,36 @@ Python face of the reference's C++ class (cpp/src/cuda/kernel.h:64-151,
 bindings cpp/src/frontend/model_bindings.cpp:57-82).  `MeasuredKernel` and
 `PredictedKernel` follow analyzer/habitat/analysis/kernels.py:3-44.
 """
+import struct
+
+from habitat_amd.analysis.metrics import Metric
+
+# hbt_kernel_record (include/habitat_mi.h): num_blocks, block_size, dynamic_smem,
+# static_smem, regs, dest_regs, has_metrics, reserved; run_time_ns,
+# flop_sp_efficiency, dram_read_bytes, dram_write_bytes.
+RECORD_STRUCT = struct.Struct("<8i4d")
+_ROOFLINE_METRICS = (Metric.SinglePrecisionFLOPEfficiency, Metric.DRAMReadBytes,
+                     Metric.DRAMWriteBytes)
+
+
+def pack_record(kernel):
+    """(64-byte hbt_kernel_record of `kernel` with dest_regs = -1, has_metrics)
+    for any object with the reference's kernel interface."""
+    fast = getattr(kernel, "launch_fields", None)
+    if fast is not None:
+        nb, block, dyn, stat, regs, t_ns = fast()
+    else:
+        md = kernel.metadata
+        nb, block, dyn, stat, regs, t_ns = (
+            kernel.num_blocks, md["block_size"], md["dynamic_shared_memory"],
+            md["static_shared_memory"], md["registers_per_thread"], kernel.run_time_ns)
+    try:
+        eff, rd, wr = [kernel.get_metric(m) for m in _ROOFLINE_METRICS]
+        has = 1
+    except AttributeError:
+        eff = rd = wr = 0.0
+        has = 0
+    return RECORD_STRUCT.pack(nb, block, dyn, stat, regs, -1, has, 0, t_ns, eff, rd, wr), has
 
 
 class KernelInstance:
@@ -70,6 +100,7 @@ class MeasuredKernel:
         self._metrics_kernels = metrics_kernels
         self._device = device
         self._cached_metrics = {}
+        self._packed = None
 
     def get_metric(self, metric_info, default=None):
         if metric_info in self._cached_metrics:
@@ -94,6 +125,22 @@ class MeasuredKernel:
     def launch_fields(self):
         return self._c.launch_fields()
 
+    def packed_record(self):
+        """(this kernel as a 64-byte hbt_kernel_record with dest_regs = -1, whether
+        it has the three roofline metrics).  Built on first use and kept: the
+        launch fields cannot change through this interface and a metric, once
+        read, is cached for good (`_cached_metrics`, as in the reference); only
+        a kernel found WITHOUT its metrics is looked at again when raw metrics
+        have been added to its metric kernels since."""
+        packed = self._packed
+        if packed is not None:
+            if packed[1] or packed[2] == sum(len(k.metrics) for k in self._metrics_kernels):
+                return packed
+        record, has = pack_record(self)
+        self._packed = packed = (record, has,
+                                 sum(len(k.metrics) for k in self._metrics_kernels))
+        return packed
+
     def __getattr__(self, name):
         # Everything else comes from the underlying kernel instance.
         if name == "_c":
@@ -102,6 +149,8 @@ class MeasuredKernel:
 
 
 class PredictedKernel:
+    __slots__ = ("_measured_kernel", "_run_time_ns")
+
     def __init__(self, measured_kernel, run_time_ns):
         self._measured_kernel = measured_kernel
         self._run_time_ns = run_time_ns

@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libhabitat_mi.so")
 
-SOURCES = ["api.hip", "wave_scale.hip", "mlp.hip", "trace.hip", "device_info.hip"]
+SOURCES = ["api.hip", "host_records.hip", "wave_scale.hip", "mlp.hip", "trace.hip", "device_info.hip"]
 
 # -packed-fp32-ops is switched OFF: the compiler must not form v_pk_*_f32.
 HIPCC_FLAGS = [

@@ -1,11 +1,9 @@
 // C ABI of the library (include/habitat_mi.h): argument checking, host-side
-// folding of device constants, launches.  No allocation happens here except in
-// hbt_mlp_create (mlp.hip).
+// folding of device constants, launches.  No allocation happens here.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
 #include <cstdint>
-#include <mutex>
 
 #include "../../include/habitat_mi.h"
 #include "occupancy.h"
@@ -210,83 +208,6 @@ int hbt_wave_scale(const hbt_device_spec* origin, const hbt_device_spec* dests, 
     }
     if (launch_wave_scale(a, vec, stream) != hipSuccess) return HBT_EHIP;
   }
-  return HBT_OK;
-}
-
-namespace {
-
-// Pinned, device-visible staging of hbt_wave_scale_one, one block per HIP
-// device, allocated on first use and kept until the process ends: 64 bytes of
-// record, 24 bytes of result (offsets in hbt_wave_scale_one).
-struct OneStaging {
-  std::mutex lock;   // one call at a time per device: the block is shared
-  unsigned char* host = nullptr;
-  unsigned char* device = nullptr;
-};
-constexpr int kMaxOneDevices = 64;
-OneStaging g_one[kMaxOneDevices];
-
-}  // namespace
-
-int hbt_wave_scale_one(const hbt_device_spec* origin, const hbt_device_spec* dest,
-                       const hbt_kernel_record* record, double* out_time_ns,
-                       int32_t* out_occ_origin, int32_t* out_occ_dest, uint8_t* out_status,
-                       void* hip_stream) {
-  if (origin == nullptr || dest == nullptr || record == nullptr || out_time_ns == nullptr ||
-      out_status == nullptr)
-    return HBT_EINVAL;
-  int rc = hbt_device_spec_check(origin);
-  if (rc == HBT_OK) rc = hbt_device_spec_check(dest);
-  if (rc != HBT_OK) return rc;
-  int device = -1;
-  if (hipGetDevice(&device) != hipSuccess) {
-    (void)hipGetLastError();
-    return HBT_EHIP;
-  }
-  if (device < 0 || device >= kMaxOneDevices) return HBT_ESIZE;
-  OneStaging& st = g_one[device];
-  std::lock_guard<std::mutex> guard(st.lock);
-  if (st.host == nullptr) {
-    void* h = nullptr;
-    void* d = nullptr;
-    if (hipHostMalloc(&h, 128, hipHostMallocDefault) != hipSuccess ||
-        hipHostGetDevicePointer(&d, h, 0) != hipSuccess || d == nullptr) {
-      (void)hipGetLastError();
-      if (h != nullptr) (void)hipHostFree(h);
-      return HBT_ENOMEM;
-    }
-    st.host = static_cast<unsigned char*>(h);
-    st.device = static_cast<unsigned char*>(d);
-  }
-  // record: 0 t, 8 eff, 16 read, 24 written (fp64); 32 num_blocks, 36 block, 40
-  // dynamic, 44 static, 48 regs, 52 dest_regs (int32); 56 has_metrics (uint8).
-  // result at 64: time (fp64); 72 origin occupancy, 76 destination occupancy
-  // (int32); 80 status (uint8).
-  double* f64 = reinterpret_cast<double*>(st.host);
-  int32_t* i32 = reinterpret_cast<int32_t*>(st.host + 32);
-  f64[0] = record->run_time_ns; f64[1] = record->flop_sp_efficiency;
-  f64[2] = record->dram_read_bytes; f64[3] = record->dram_write_bytes;
-  i32[0] = record->num_blocks; i32[1] = record->block_size; i32[2] = record->dynamic_smem;
-  i32[3] = record->static_smem; i32[4] = record->regs; i32[5] = record->dest_regs;
-  st.host[56] = record->has_metrics != 0 ? 1 : 0;
-  unsigned char* d = st.device;
-  rc = hbt_wave_scale(origin, dest, 1, 1, reinterpret_cast<int32_t*>(d + 32),
-                      reinterpret_cast<int32_t*>(d + 36), reinterpret_cast<int32_t*>(d + 40),
-                      reinterpret_cast<int32_t*>(d + 44), reinterpret_cast<int32_t*>(d + 48),
-                      reinterpret_cast<int32_t*>(d + 52), reinterpret_cast<double*>(d),
-                      reinterpret_cast<double*>(d + 8), reinterpret_cast<double*>(d + 16),
-                      reinterpret_cast<double*>(d + 24), d + 56, reinterpret_cast<double*>(d + 64),
-                      reinterpret_cast<int32_t*>(d + 72), reinterpret_cast<int32_t*>(d + 76),
-                      nullptr, nullptr, d + 80, hip_stream);
-  if (rc != HBT_OK) return rc;
-  if (hipStreamSynchronize(static_cast<hipStream_t>(hip_stream)) != hipSuccess) {
-    (void)hipGetLastError();
-    return HBT_EHIP;
-  }
-  *out_time_ns = *reinterpret_cast<const double*>(st.host + 64);
-  if (out_occ_origin != nullptr) *out_occ_origin = *reinterpret_cast<const int32_t*>(st.host + 72);
-  if (out_occ_dest != nullptr) *out_occ_dest = *reinterpret_cast<const int32_t*>(st.host + 76);
-  *out_status = st.host[80];
   return HBT_OK;
 }
 

@@ -1,0 +1,210 @@
+// Wave scaling of kernel records that live in HOST memory as an array of
+// structures, results back in host memory: the boundary for callers that hold
+// Python (or C++) kernel objects rather than columns on the GPU.
+//
+//   hbt_wave_scale_host_records   n records, one destination, one call: the
+//       reference's per-kernel loop of Predictor._wave_scale
+//       (analyzer/habitat/analysis/predictor.py:116-124) over the kernels of a
+//       pass, an operation or a whole trace.
+//   hbt_wave_scale_one            the same for one record: one call of the
+//       strategy signature (wave_scaling/unified.py:8-35).
+//
+// Records and results travel through a pinned, device-visible staging block the
+// library keeps per GPU (allocated on the first call there, kept until the
+// process ends); the kernel reads the records and writes the results straight
+// through it, so a call is one memcpy into the block, one launch, one wait and
+// one memcpy out.  The arithmetic is the code of wave_scale_device.h that the
+// column kernel runs.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstring>
+#include <mutex>
+
+#include "../../include/habitat_mi.h"
+#include "occupancy.h"
+#include "wave_scale.h"
+
+#pragma clang fp contract(off)
+
+#include "wave_scale_device.h"
+
+namespace hbt {
+namespace {
+
+using namespace dev;
+
+constexpr int kBlock = 256;
+// Records per pass through the staging block; longer arrays take several passes.
+constexpr int64_t kChunk = 16384;
+
+static_assert(sizeof(hbt_kernel_record) == 64, "the kernel reads a record as four 16-byte loads");
+
+struct HostRecordArgs {
+  int64_t n;
+  const hbt_kernel_record* rec;  // device-visible host memory
+  double* time_ns;
+  int32_t* occ_origin;
+  int32_t* occ_dest;
+  uint8_t* status;
+  OriginArgs origin;
+  DestArgs dest;
+};
+
+using i32x4 = int32_t __attribute__((ext_vector_type(4)));
+using f64x2 = double __attribute__((ext_vector_type(2)));
+
+// One thread per record.
+template <int MODEL>
+__global__ __launch_bounds__(kBlock) void wave_scale_records_kernel(const HostRecordArgs a) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= a.n) return;
+  const char* p = reinterpret_cast<const char*>(a.rec + i);
+  const i32x4 q0 = *reinterpret_cast<const i32x4*>(p);
+  const i32x4 q1 = *reinterpret_cast<const i32x4*>(p + 16);
+  const f64x2 d0 = *reinterpret_cast<const f64x2*>(p + 32);
+  const f64x2 d1 = *reinterpret_cast<const f64x2*>(p + 48);
+  RecordIn r;
+  r.nb = q0[0];
+  r.block = q0[1];
+  r.smem_total = smem_sum(q0[3], q0[2]);
+  r.regs = q1[0];
+  r.dest_regs = q1[1];
+  r.metrics = q1[2] != 0;
+  r.t = d0[0];
+  r.eff = d0[1];
+  r.rd = d1[0];
+  r.wr = d1[1];
+
+  RecordMid m = origin_part<MODEL>(a.origin, r);
+  if (__builtin_expect(m.redo_gflops, 0))
+    m.num_gflops = origin_gflops_exact(a.origin.peak_gflops, r.eff, r.t);
+  RecordOut o = dest_part<MODEL, false>(a.dest, r, m, 0.0);
+  if (__builtin_expect(o.in_order, 0))
+    o.t = scaled_time_in_order(r.t, o.gamma, a.dest.log2_bw, a.dest.log2_clk, a.dest.log2_clk_sm);
+  a.time_ns[i] = o.t;
+  a.occ_origin[i] = m.occ_o;
+  a.occ_dest[i] = o.occ_d;
+  a.status[i] = o.status;
+}
+
+// The staging block of one GPU: kChunk records in, their results out.
+struct Staging {
+  std::mutex lock;  // one call at a time per device: the block is shared
+  unsigned char* host = nullptr;
+  unsigned char* device = nullptr;
+};
+constexpr size_t kOffTime = (size_t)kChunk * sizeof(hbt_kernel_record);
+constexpr size_t kOffOccOrigin = kOffTime + (size_t)kChunk * sizeof(double);
+constexpr size_t kOffOccDest = kOffOccOrigin + (size_t)kChunk * sizeof(int32_t);
+constexpr size_t kOffStatus = kOffOccDest + (size_t)kChunk * sizeof(int32_t);
+constexpr size_t kStagingBytes = kOffStatus + (size_t)kChunk;
+constexpr int kMaxDevices = 64;
+Staging g_staging[kMaxDevices];
+
+int staging_ready(Staging& st) {
+  if (st.host != nullptr) return HBT_OK;
+  void* h = nullptr;
+  void* d = nullptr;
+  if (hipHostMalloc(&h, kStagingBytes, hipHostMallocDefault) != hipSuccess ||
+      hipHostGetDevicePointer(&d, h, 0) != hipSuccess || d == nullptr) {
+    (void)hipGetLastError();
+    if (h != nullptr) (void)hipHostFree(h);
+    return HBT_ENOMEM;
+  }
+  st.host = static_cast<unsigned char*>(h);
+  st.device = static_cast<unsigned char*>(d);
+  return HBT_OK;
+}
+
+// The stream must be usable for a launch followed by a wait: not under
+// capture, and a stream of the current device (whose staging block is used).
+int stream_usable(hipStream_t stream, int device) {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+    (void)hipGetLastError();
+    return HBT_EHIP;
+  }
+  if (capture != hipStreamCaptureStatusNone) return HBT_EINVAL;
+  hipDevice_t of_stream = device;
+  if (hipStreamGetDevice(stream, &of_stream) == hipSuccess) {
+    if ((int)of_stream != device) return HBT_EINVAL;
+  } else {
+    (void)hipGetLastError();
+  }
+  return HBT_OK;
+}
+
+}  // namespace
+}  // namespace hbt
+
+extern "C" {
+
+int hbt_wave_scale_host_records(const hbt_device_spec* origin, const hbt_device_spec* dest,
+                                int64_t n, const hbt_kernel_record* records, double* out_time_ns,
+                                uint8_t* out_status, int32_t* out_occ_origin,
+                                int32_t* out_occ_dest, void* hip_stream) {
+  using namespace hbt;
+  if (origin == nullptr || dest == nullptr || n < 0) return HBT_EINVAL;
+  int rc = hbt_device_spec_check(origin);
+  if (rc == HBT_OK) rc = hbt_device_spec_check(dest);
+  if (rc != HBT_OK) return rc;
+  if (n == 0) return HBT_OK;
+  if (records == nullptr || out_time_ns == nullptr || out_status == nullptr) return HBT_EINVAL;
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    return HBT_EHIP;
+  }
+  if (device < 0 || device >= kMaxDevices) return HBT_ESIZE;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  if ((rc = stream_usable(stream, device)) != HBT_OK) return rc;
+
+  Staging& st = g_staging[device];
+  std::lock_guard<std::mutex> guard(st.lock);
+  if ((rc = staging_ready(st)) != HBT_OK) return rc;
+
+  HostRecordArgs a{};
+  a.rec = reinterpret_cast<const hbt_kernel_record*>(st.device);
+  a.time_ns = reinterpret_cast<double*>(st.device + kOffTime);
+  a.occ_origin = reinterpret_cast<int32_t*>(st.device + kOffOccOrigin);
+  a.occ_dest = reinterpret_cast<int32_t*>(st.device + kOffOccDest);
+  a.status = st.device + kOffStatus;
+  a.origin = make_origin_args(*origin);
+  a.dest = make_dest_args(*origin, *dest);
+  const int model = dev::model_for(a.origin.dev, &a.dest, 1);
+
+  for (int64_t done = 0; done < n; done += kChunk) {
+    const int64_t m = (n - done < kChunk) ? (n - done) : kChunk;
+    std::memcpy(st.host, records + done, (size_t)m * sizeof(hbt_kernel_record));
+    a.n = m;
+    const dim3 grid((unsigned)((m + kBlock - 1) / kBlock));
+    dev::with_model(model, [&](auto mc) {
+      hipLaunchKernelGGL(wave_scale_records_kernel<decltype(mc)::value>, grid, dim3(kBlock), 0,
+                         stream, a);
+    });
+    if (hipGetLastError() != hipSuccess) return HBT_EHIP;
+    if (hipStreamSynchronize(stream) != hipSuccess) {
+      (void)hipGetLastError();
+      return HBT_EHIP;
+    }
+    std::memcpy(out_time_ns + done, st.host + kOffTime, (size_t)m * sizeof(double));
+    std::memcpy(out_status + done, st.host + kOffStatus, (size_t)m);
+    if (out_occ_origin != nullptr)
+      std::memcpy(out_occ_origin + done, st.host + kOffOccOrigin, (size_t)m * sizeof(int32_t));
+    if (out_occ_dest != nullptr)
+      std::memcpy(out_occ_dest + done, st.host + kOffOccDest, (size_t)m * sizeof(int32_t));
+  }
+  return HBT_OK;
+}
+
+int hbt_wave_scale_one(const hbt_device_spec* origin, const hbt_device_spec* dest,
+                       const hbt_kernel_record* record, double* out_time_ns,
+                       int32_t* out_occ_origin, int32_t* out_occ_dest, uint8_t* out_status,
+                       void* hip_stream) {
+  if (record == nullptr || out_time_ns == nullptr || out_status == nullptr) return HBT_EINVAL;
+  return hbt_wave_scale_host_records(origin, dest, 1, record, out_time_ns, out_status,
+                                     out_occ_origin, out_occ_dest, hip_stream);
+}
+
+}  // extern "C"

@@ -10,7 +10,7 @@
  * without a GPU the compute entry points return HBT_EHIP.  Only the two
  * *_create calls allocate device memory (and the calibration calls at the
  * end, which say so); the library's only state outside its handles is what
- * hbt_wave_scale_one and hbt_mlp_forward_static say they keep per GPU.
+ * hbt_wave_scale_host_records and hbt_mlp_forward_static say they keep per GPU.
  *
  * Each entry point cites the reference interface it stands in for
  * (paths relative to the reference tree).
@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define HBT_VERSION 102 /* 0.1.2 */
+#define HBT_VERSION 103 /* 0.1.3 */
 
 enum {
   HBT_OK = 0,
@@ -161,26 +161,42 @@ int hbt_wave_scale(const hbt_device_spec *origin, const hbt_device_spec *dests, 
                    void *hip_stream);
 
 /*
- * One kernel record, one destination, start to finish: the reference's strategy
- * call  strategy(kernel, origin_device, dest_device, metadata_manager)
- * (analysis/predictor.py:116-124 invoking wave_scaling/unified.py:8-35) as one C
- * call.  `record` and the out pointers are HOST memory.  The record goes through
- * a pinned, device-visible staging block of the library (128 bytes per GPU,
- * allocated on the first call there and kept), the same kernel as
- * hbt_wave_scale runs on it on `hip_stream`, and the call waits for the stream
- * before it returns: some 15 us, all of it launch and wait (21 us per kernel
- * through the Python strategy that wraps it).  dest_regs < 0 =
- * no register-table entry; has_metrics == 0 selects the no-metrics strategy.
- * *out_status is one of HBT_ST_*; the time is NaN unless it is HBT_ST_OK.
- * out_occ_origin and out_occ_dest are nullable.  Calls on one GPU are
- * serialised inside the library.  Callers with many kernels should hand them
- * over together (hbt_wave_scale).
+ * Kernel records held in HOST memory as an array of structures, one
+ * destination, results back in host memory, start to finish: the per-kernel
+ * loop of Predictor._wave_scale (analysis/predictor.py:116-124), i.e. n calls of
+ * strategy(kernel, origin_device, dest_device, metadata_manager)
+ * (wave_scaling/unified.py:8-35), as ONE C call.  This is the entry for callers
+ * that hold kernel objects on the host (the reference's plug point) rather
+ * than columns on the GPU.  `records`, out_time_ns [n], out_status [n],
+ * out_occ_origin [n] and out_occ_dest [n] (both nullable) are HOST memory.
+ * Per record: dest_regs < 0 = no register-table entry; has_metrics == 0 selects
+ * the no-metrics strategy; out_status is one of HBT_ST_* and the time is NaN
+ * unless it is HBT_ST_OK.
+ *
+ * The records go through a pinned, device-visible staging block of the library
+ * (about 1.3 MiB per GPU, allocated on the first call there and kept), in passes
+ * of 16384 records; per pass one launch on `hip_stream` and a wait for the
+ * stream, so the call returns with the results in place (some 15 us for up to a
+ * few thousand records).  Calls on one GPU are serialised inside the library.
+ * `hip_stream` must be a stream of the current device and must not be under
+ * graph capture (HBT_EINVAL): the call waits for it.
  */
 typedef struct hbt_kernel_record {
   int32_t num_blocks, block_size, dynamic_smem, static_smem, regs, dest_regs;
   int32_t has_metrics, reserved;
   double run_time_ns, flop_sp_efficiency, dram_read_bytes, dram_write_bytes;
 } hbt_kernel_record;
+int hbt_wave_scale_host_records(const hbt_device_spec *origin, const hbt_device_spec *dest,
+                                int64_t n, const hbt_kernel_record *records, double *out_time_ns,
+                                uint8_t *out_status, int32_t *out_occ_origin,
+                                int32_t *out_occ_dest, void *hip_stream);
+
+/*
+ * One kernel record: hbt_wave_scale_host_records with n = 1, the reference's
+ * strategy call (analysis/predictor.py:116-124 invoking
+ * wave_scaling/unified.py:8-35) one kernel at a time.  All of its cost is the
+ * launch and the wait; callers with many kernels should hand them over together.
+ */
 int hbt_wave_scale_one(const hbt_device_spec *origin, const hbt_device_spec *dest,
                        const hbt_kernel_record *record, double *out_time_ns,
                        int32_t *out_occ_origin, int32_t *out_occ_dest, uint8_t *out_status,

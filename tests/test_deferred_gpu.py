@@ -1,0 +1,273 @@
+"""GPU: kernel records handed over from host memory (hbt_wave_scale_host_records)
+and the deferred strategies built on it, which keep the reference's one-call-
+per-kernel plug point (predictor.py:116-124) at one launch per trace."""
+import ctypes
+import threading
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import oracle_device
+from habitat_amd import Device, _lib, synthetic
+from habitat_amd.analysis.kernels import PredictedKernel
+from habitat_amd.analysis.predictor import Predictor
+from habitat_amd.analysis.wave_scaling import deferred
+from habitat_amd.analysis.wave_scaling.batch import KernelRecords, wave_scale
+from habitat_amd.analysis.wave_scaling.deferred import (
+    RECORD_DTYPE, deferred_resimplified_wave_scaling, deferred_roofline_wave_scaling,
+    deferred_unified_wave_scaling)
+from habitat_amd.analysis.wave_scaling.metadata import NullMetadataManager
+from habitat_amd.analysis.wave_scaling.unified import unified_wave_scaling
+from oracle import lib as olib
+from test_api_gpu import (TableManager, make_kernel, oracle_operation_ms, seeded_predictors)
+
+pytestmark = pytest.mark.gpu
+
+TIME_RTOL = 1e-6
+
+
+def odev(d):
+    return oracle_device(d.as_dict())
+
+
+def host_records(rec):
+    """numpy columns -> array of hbt_kernel_record."""
+    n = rec["num_blocks"].shape[0]
+    out = np.zeros(n, RECORD_DTYPE)
+    out["num_blocks"], out["block_size"] = rec["num_blocks"], rec["block_size"]
+    out["dynamic_smem"], out["static_smem"] = rec["dynamic_smem"], rec["static_smem"]
+    out["regs"] = rec["regs_per_thread"]
+    out["dest_regs"] = rec.get("dest_regs", np.full(n, -1, np.int32))
+    out["has_metrics"] = rec.get("has_metrics", np.ones(n, np.uint8))
+    for name in ("run_time_ns", "flop_sp_efficiency", "dram_read_bytes", "dram_write_bytes"):
+        out[name] = rec[name]
+    return out
+
+
+def call_host_records(origin, dest, records, stream=None, occupancies=True):
+    n = records.shape[0]
+    t = np.full(n, -1.0)
+    st = np.full(n, 255, np.uint8)
+    oo = np.full(n, -1, np.int32)
+    od = np.full(n, -1, np.int32)
+    p = lambda a: ctypes.c_void_p(a.ctypes.data)
+    stream = stream or torch.cuda.current_stream()
+    rc = _lib.lib().hbt_wave_scale_host_records(
+        ctypes.byref(origin.spec), ctypes.byref(dest.spec), n, p(records), p(t), p(st),
+        p(oo) if occupancies else None, p(od) if occupancies else None,
+        ctypes.c_void_p(stream.cuda_stream))
+    return rc, t, st, oo, od
+
+
+@pytest.mark.parametrize("n", [1, 63, 257, 10_000, 16_384, 16_385, 40_000])
+def test_host_records_match_the_oracle_and_the_column_kernel(n):
+    """configs[0]'s records (10 000 of them among the sizes) as host structures:
+    one pass through the staging block, exactly one, and three."""
+    origin, dest = Device.V100, Device.MI355X
+    rec, _ = synthetic.kernel_records(n, origin, seed=n)
+    rng = np.random.default_rng(n)
+    rec["has_metrics"] = (rng.random(n) < 0.7).astype(np.uint8)
+    rec["dest_regs"] = np.where(rng.random(n) < 0.3, rng.integers(16, 200, n), -1).astype(np.int32)
+    rc, t, st, oo, od = call_host_records(origin, dest, host_records(rec))
+    assert rc == 0
+    want = olib.wave_scale(odev(origin), odev(dest), rec)
+    assert np.array_equal(oo, want["occ_origin"]) and np.array_equal(od, want["occ_dest"])
+    assert np.array_equal(st, want["status"])
+    ok = want["status"] == 0
+    assert np.all(np.isnan(t[~ok]))
+    np.testing.assert_allclose(t[ok], want["time_ns"][ok], rtol=TIME_RTOL)
+    err = np.max(np.abs(t[ok] - want["time_ns"][ok]) / np.abs(want["time_ns"][ok]))
+    print("host records n=%d: max relative time error vs oracle %.3g" % (n, err))
+    # the same arithmetic as the column kernel: bit for bit
+    out = wave_scale(KernelRecords.from_numpy(rec), origin, [dest])
+    assert np.array_equal(out.time_ns[0].cpu().numpy(), t, equal_nan=True)
+    assert np.array_equal(out.status[0].cpu().numpy(), st)
+
+
+def test_host_records_arguments_and_streams():
+    origin, dest = Device.V100, Device.T4
+    lib = _lib.lib()
+    rec, _ = synthetic.kernel_records(300, origin, seed=1)
+    records = host_records(rec)
+    rc, t, st, _, _ = call_host_records(origin, dest, records, occupancies=False)
+    assert rc == 0 and st.max() < 255 and np.all(t[st == 0] > 0)
+    side = torch.cuda.Stream()
+    rc2, t2, st2, _, _ = call_host_records(origin, dest, records, stream=side)
+    assert rc2 == 0 and np.array_equal(t, t2, equal_nan=True) and np.array_equal(st, st2)
+    # nothing to do, and what must be refused
+    o, d = ctypes.byref(origin.spec), ctypes.byref(dest.spec)
+    assert lib.hbt_wave_scale_host_records(o, d, 0, None, None, None, None, None, None) == 0
+    assert lib.hbt_wave_scale_host_records(o, d, -1, None, None, None, None, None, None) == _lib.HBT_EINVAL
+    assert lib.hbt_wave_scale_host_records(o, d, 5, None, None, None, None, None, None) == _lib.HBT_EINVAL
+    assert lib.hbt_wave_scale_host_records(None, d, 0, None, None, None, None, None, None) == _lib.HBT_EINVAL
+    bad = _lib.DeviceSpec.from_buffer_copy(dest.spec)
+    bad.mem_bandwidth_gb = 0.0
+    assert lib.hbt_wave_scale_host_records(o, ctypes.byref(bad), 0, None, None, None, None, None,
+                                           None) == _lib.HBT_ESPEC
+
+
+def test_a_capturing_stream_is_refused_and_the_capture_survives():
+    """The call waits for its stream, which a stream under graph capture cannot
+    do: it is refused before anything is launched, and the capture goes on."""
+    origin, dest = Device.V100, Device.T4
+    rec, _ = synthetic.kernel_records(8, origin, seed=2)
+    records = host_records(rec)
+    call_host_records(origin, dest, records)            # staging exists before the capture
+    x = torch.zeros(16, device="cuda")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc, _, st, _, _ = call_host_records(origin, dest, records)
+        x.add_(1.0)
+    assert rc == _lib.HBT_EINVAL and np.all(st == 255)
+    graph.replay()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert float(x[0]) == 2.0
+    rc, _, st, _, _ = call_host_records(origin, dest, records)
+    assert rc == 0 and st.max() < 255
+
+
+def test_deferred_strategies_known_answers(kat):
+    mm = NullMetadataManager()
+    for row in kat["scaling"]:
+        o, d = getattr(Device, row["origin"]), getattr(Device, row["dest"])
+        over = row.get("record", {})
+        metrics = (over.get("flop_sp_efficiency", 50.0), 1e8, 1e8)
+        has_metrics = row.get("has_metrics", True)
+        k = make_kernel(o, num_blocks=row["num_blocks"], metrics=metrics if has_metrics else None)
+        manager = mm if "dest_regs" not in row else TableManager({("k", d.name): row["dest_regs"]})
+        strategies = ((deferred_unified_wave_scaling, deferred_roofline_wave_scaling) if has_metrics
+                      else (deferred_unified_wave_scaling, deferred_resimplified_wave_scaling))
+        for strategy in strategies:
+            p = strategy(k, o, d, manager)
+            assert isinstance(p, PredictedKernel) and p.name == "k"
+            assert deferred.pending_kernels() == 1
+            assert p.run_time_ns == pytest.approx(row["time_ns"], rel=TIME_RTOL)
+            assert deferred.pending_kernels() == 0
+    k = make_kernel(Device.V100, metrics=None)
+    with pytest.raises(AttributeError, match="Unknown metric"):     # in the call, as the reference
+        deferred_roofline_wave_scaling(k, Device.V100, Device.P100, mm)
+    assert deferred_unified_wave_scaling(k, Device.V100, Device.P100, mm).run_time_ns == \
+        pytest.approx(1e6 * 739 / 501, rel=1e-12)
+    small = make_kernel(Device.V100, num_blocks=3, metrics=None)
+    t = deferred_resimplified_wave_scaling(small, Device.V100, Device.P100, mm).run_time_ns
+    assert t == 1000000 and isinstance(t, int)          # the measured value itself
+
+
+def test_deferred_exceptions_surface_at_the_read_in_the_reference_s_order():
+    mm = NullMetadataManager()
+    v100, p100 = Device.V100, Device.P100
+    kernels = [make_kernel(v100, 5000, name="fine0"),
+               make_kernel(v100, 100, metrics=(50.0, -3e8, 1e8), name="gamma"),   # AssertionError
+               make_kernel(v100, 7000, name="fine1"),
+               make_kernel(v100, 100, 1024, regs=255, name="origin0"),            # ZeroDivisionError
+               make_kernel(v100, 0, name="blocks0")]                              # ZeroDivisionError
+    preds = [deferred_unified_wave_scaling(k, v100, p100, mm) for k in kernels]   # nothing raised
+    assert deferred.pending_kernels() == 5
+    eager = []
+    for k in kernels:
+        try:
+            eager.append(unified_wave_scaling(k, v100, p100, mm).run_time_ns)
+        except (ZeroDivisionError, AssertionError) as exc:
+            eager.append(type(exc))
+    assert eager[1] is AssertionError and eager[3] is ZeroDivisionError and eager[4] is ZeroDivisionError
+    for p, want in zip(preds, eager):
+        if isinstance(want, type):
+            for _ in range(2):                   # on every read
+                with pytest.raises(want):
+                    p.run_time_ns
+        else:
+            assert p.run_time_ns == want         # same kernel code: bit for bit
+    # the reference's sum over a pass (run_time.py:50-58) stops at the first of them
+    with pytest.raises(AssertionError):
+        sum(map(lambda k: k.run_time_ns, preds))
+    with pytest.raises(ZeroDivisionError):
+        sum(map(lambda k: k.run_time_ns, preds[2:]))
+
+
+def test_deferred_strategy_through_the_predictor_on_the_resnet50_trace():
+    """The reference's loop shape: Trace.to_device -> Predictor.predict_operation per
+    operation -> strategy per kernel (predictor.py:116-124), read afterwards
+    (run_time.py:50-58).  With the deferred strategy nothing is launched until
+    the first read, and that read hands over every kernel of the trace."""
+    origin, dest = Device.V100, Device.T4
+    trace = synthetic.resnet50_trace(origin, batch=32, seed=3)
+    preds = seeded_predictors()
+    n_kernels = sum(len(rt.kernels) for op in trace.operations
+                    for rt in (op.forward, op.backward) if rt is not None)
+    assert n_kernels >= 800
+    predictor = Predictor(mlp_predictors=preds, wave_scaling_strategy=deferred_unified_wave_scaling)
+    predicted = trace.to_device(dest, predictor)
+    assert deferred.pending_kernels() == n_kernels          # one set, nothing launched yet
+    scaled = [op for op in predicted.operations if op.name not in ("conv2d", "linear")]
+    first = scaled[0].forward.kernels[0]
+    pending = first._set
+    assert pending.times is None
+    first.run_time_ns                                        # the first read ...
+    assert deferred.pending_kernels() == 0 and len(pending.times) == n_kernels   # ... hands over all
+    want = [oracle_operation_ms(op, dest, preds) for op in trace.operations]
+    got = [op.run_time_ms for op in predicted.operations]
+    worst = 0.0
+    for op, g, w in zip(trace.operations, got, want):
+        tol = 1e-4 if op.name in ("conv2d", "linear") else TIME_RTOL
+        assert g == pytest.approx(w, rel=tol), op.name
+        if op.name not in ("conv2d", "linear"):
+            worst = max(worst, abs(g - w) / abs(w))
+    print("deferred strategy, %d kernels: max relative error of a wave-scaled operation vs the "
+          "oracle %.3g" % (n_kernels, worst))
+    # and the batched built-in path gives the same kernel times, bit for bit
+    builtin = trace.to_device(dest, Predictor(mlp_predictors=preds))
+    for a, b in zip(predicted.operations, builtin.operations):
+        if a.name in ("conv2d", "linear"):
+            continue
+        for ra, rb in ((a.forward, b.forward), (a.backward, b.backward)):
+            if ra is not None:
+                assert [k.run_time_ns for k in ra.kernels] == [k.run_time_ns for k in rb.kernels]
+    # a second destination starts a second set; the first keeps its results
+    other = trace.to_device(Device.P100, predictor)
+    assert deferred.pending_kernels() == n_kernels
+    assert other.run_time_ms != pytest.approx(predicted.run_time_ms, rel=1e-3)
+    assert [op.run_time_ms for op in predicted.operations] == got
+
+
+def test_deferred_sets_are_per_thread_and_use_the_register_table():
+    origin, dest = Device.V100, Device.P100
+    k = make_kernel(origin, num_blocks=400, name="gemm")
+    table = TableManager({("gemm", "P100"): 128})
+    with_table = deferred_unified_wave_scaling(k, origin, dest, table)
+    without = deferred_unified_wave_scaling(k, origin, dest, NullMetadataManager())  # another set
+    assert with_table._set is not without._set
+    assert with_table.run_time_ns == unified_wave_scaling(k, origin, dest, table).run_time_ns
+    assert without.run_time_ns == unified_wave_scaling(k, origin, dest,
+                                                       NullMetadataManager()).run_time_ns
+    assert with_table.run_time_ns != without.run_time_ns
+
+    mm = NullMetadataManager()
+    kernels = [make_kernel(origin, num_blocks=64 + 997 * i, t_ns=1_000_000 + 12_345 * i,
+                           metrics=(10.0 + i, 1e8, 2e8) if i % 3 else None) for i in range(64)]
+    want = [unified_wave_scaling(kk, origin, Device.T4, mm).run_time_ns for kk in kernels]
+    got = [None] * len(kernels)
+    errors = []
+
+    def work(start):
+        try:
+            torch.cuda.set_device(0)
+            for _ in range(5):
+                mine = list(range(start, len(kernels), 4))
+                preds = [deferred_unified_wave_scaling(kernels[i], origin, Device.T4, mm)
+                         for i in mine]
+                assert deferred.pending_kernels() == len(mine)
+                for i, p in zip(mine, preds):
+                    got[i] = p.run_time_ns
+        except Exception as exc:       # noqa: BLE001 - reported below
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert got == want
