@@ -2,8 +2,11 @@
 // folding of device constants, launches.  No allocation happens here.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
+#include <cstring>
+#include <vector>
 
 #include "../../include/habitat_mi.h"
 #include "occupancy.h"
@@ -33,6 +36,45 @@ DestArgs make_dest_args(const hbt_device_spec& o, const hbt_device_spec& d) {
   p.log2_clk = std::log2(clk_ratio);
   p.log2_clk_sm = p.log2_clk + std::log2(sm_ratio);
   return p;
+}
+
+static bool same_occupancy_constants(OccDevice a, OccDevice b) {
+  a.num_sms = b.num_sms = 0;
+  a.flags &= ~kSameOccAsPrev;
+  b.flags &= ~kSameOccAsPrev;
+  return std::memcmp(&a, &b, sizeof(OccDevice)) == 0;
+}
+
+void group_by_occupancy(DestArgs* dests, int32_t* order, int n) {
+  if (n <= 1) {
+    if (n == 1) {
+      order[0] = 0;
+      dests[0].dev.flags &= ~kSameOccAsPrev;
+    }
+    return;
+  }
+  // class of a destination = position of the first one with its constants;
+  // a stable sort by class keeps the caller's order within a class
+  std::vector<int32_t> cls((size_t)n);
+  for (int i = 0; i < n; ++i) {
+    cls[i] = i;
+    for (int j = 0; j < i; ++j)
+      if (cls[j] == j && same_occupancy_constants(dests[j].dev, dests[i].dev)) {
+        cls[i] = j;
+        break;
+      }
+  }
+  std::vector<int32_t> idx((size_t)n);
+  for (int i = 0; i < n; ++i) idx[i] = i;
+  std::stable_sort(idx.begin(), idx.end(), [&](int32_t a, int32_t b) { return cls[a] < cls[b]; });
+  std::vector<DestArgs> sorted((size_t)n);
+  for (int i = 0; i < n; ++i) {
+    sorted[i] = dests[idx[i]];
+    sorted[i].dev.flags &= ~kSameOccAsPrev;
+    if (i > 0 && cls[idx[i]] == cls[idx[i - 1]]) sorted[i].dev.flags |= kSameOccAsPrev;
+    order[i] = idx[i];
+  }
+  for (int i = 0; i < n; ++i) dests[i] = sorted[i];
 }
 
 // What make_occ_device needs: 32-bit shared-memory sizes and a bounded warp size.
@@ -193,14 +235,19 @@ int hbt_wave_scale(const hbt_device_spec* origin, const hbt_device_spec* dests, 
   a.out_occ_origin = out_occ_origin; a.out_wave_origin = out_wave_origin;
   a.origin = make_origin_args(*origin);
 
+  // Within a launch, destinations with equal occupancy constants go next to
+  // each other: the kernel evaluates the occupancy model once per run of them.
+  // Every destination keeps its own row of the outputs.
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
   for (int32_t d0 = 0; d0 < n_dest; d0 += kMaxDestPerLaunch) {
     const int32_t nd = (n_dest - d0 < kMaxDestPerLaunch) ? (n_dest - d0) : kMaxDestPerLaunch;
+    int32_t order[kMaxDestPerLaunch];
+    for (int32_t k = 0; k < nd; ++k) a.dest[k] = make_dest_args(*origin, dests[d0 + k]);
+    group_by_occupancy(a.dest, order, nd);
     a.n_dest = nd;
     a.write_origin = (d0 == 0) ? 1 : 0;
     for (int32_t k = 0; k < nd; ++k) {
-      const int64_t off = (int64_t)(d0 + k) * n;
-      a.dest[k] = make_dest_args(*origin, dests[d0 + k]);
+      const int64_t off = (int64_t)(d0 + order[k]) * n;
       a.out[k].time_ns = out_time_ns + off;
       a.out[k].occ = out_occ_dest ? out_occ_dest + off : nullptr;
       a.out[k].wave = out_wave_dest ? out_wave_dest + off : nullptr;

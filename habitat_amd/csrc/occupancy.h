@@ -44,6 +44,9 @@ enum : uint32_t {
   kPoolSteps = 1u << 5,  // cc 7.x and a block's allocation can exceed pref_pool
   kWarpPow2 = 1u << 6,   // warp_size is a power of two: warp_shift is valid
   kCdna = 1u << 7,       // AMD compute-unit model (HBT_COMPUTE_MAJOR_CDNA): occupancy_cdna
+  // Set by a launcher, not by make_occ_device: in the launch's array of
+  // destinations this one has the occupancy constants of the one before it.
+  kSameOccAsPrev = 1u << 8,
 };
 
 // Device-only constants of the occupancy model (14 dwords).  Every field fits 32 bits:

@@ -32,7 +32,16 @@ struct DestArgs {
   double log2_clk;             // log2(origin.base_clock_mhz / dest.base_clock_mhz)
   double log2_clk_sm;          // log2_clk + log2(origin.num_sms / dest.num_sms)
   float inv_sms;               // 1 / num_sms rounded to float
+
+  bool ridge_in_range() const { return ridge >= 0x1p-500 && ridge <= 0x1p500; }
 };
+
+// Puts destinations with equal occupancy constants (everything in OccDevice but
+// num_sms) next to each other and marks every destination that agrees with the
+// one before it (kSameOccAsPrev), so that a kernel walking over dests[0..n)
+// evaluates the occupancy model once per run of equal ones.  order[i] is the
+// caller's index of the destination now at position i.
+void group_by_occupancy(DestArgs* dests, int32_t* order, int n);
 
 // The origin device's share of the constants.
 struct OriginArgs {

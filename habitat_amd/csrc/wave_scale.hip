@@ -156,17 +156,38 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
 #pragma unroll
   for (int k = 0; k < R; ++k) rin[k].metrics = ((hm_bits >> (8 * k)) & 0xffu) != 0;
 
+  // With several destinations the two divisions of gamma that do not depend on
+  // the destination are made once per record (the general instantiation keeps
+  // the one-division form, which has no precondition on the ridge point).
+  constexpr bool SHARED = !SINGLE && MODEL != kModelGeneral;
+  Intensity intensity[R];
+#pragma unroll
+  for (int k = 0; k < R; ++k) {
+    finish_mid<PERMUTE>(mid[k], log2_lane);
+    if (SHARED) intensity[k] = record_intensity(mid[k].num_gflops, mid[k].total_gb);
+  }
+
   const int n_dest = SINGLE ? 1 : a.n_dest;
+  int32_t occ_d[R];
   for (int d = 0; d < n_dest; ++d) {
     const DestArgs& p = a.dest[d];
     double ot[R], gamma[R];
-    int32_t occ_d[R], wave_d[R];
+    int32_t wave_d[R];
     uint8_t st[R];
     bool in_order = false;
+    // the destination's occupancy, unless it has the constants of the one before
+    if (SINGLE || !(p.dev.flags & kSameOccAsPrev)) {
+#pragma unroll
+      for (int k = 0; k < R; ++k) occ_d[k] = dest_occupancy<MODEL>(p, rin[k], mid[k]);
+    }
 #pragma unroll
     for (int k = 0; k < R; ++k) {
-      const RecordOut o = dest_part<MODEL, PERMUTE>(p, rin[k], mid[k], log2_lane);
-      ot[k] = o.t; occ_d[k] = o.occ_d; wave_d[k] = o.wave_d; st[k] = o.status;
+      const double g =
+          SHARED ? roofline_gamma_shared(p, mid[k].num_gflops, mid[k].total_gb, intensity[k],
+                                         rin[k].metrics)
+                 : roofline_gamma(p, mid[k].num_gflops, mid[k].total_gb, rin[k].metrics);
+      const RecordOut o = dest_scale<MODEL, PERMUTE>(p, rin[k], mid[k], occ_d[k], g, log2_lane);
+      ot[k] = o.t; wave_d[k] = o.wave_d; st[k] = o.status;
       gamma[k] = o.in_order ? o.gamma : __builtin_nan("");
       in_order = in_order || o.in_order;
     }
@@ -175,7 +196,7 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
     if (w.occ != nullptr) store_r<int32_t, R>(w.occ, i, occ_d);
     if (w.wave != nullptr) store_r<int32_t, R>(w.wave, i, wave_d);
     if (w.status != nullptr) store_r<uint8_t, R>(w.status, i, st);
-    // Run times beyond 2^+-500 ns (see dest_part): the time is formed again in
+    // Run times beyond 2^+-500 ns (see dest_scale): the time is formed again in
     // the reference's order of operations and stored over the first one, after
     // everything else, where the rare call costs the other records nothing.
     if (__builtin_expect(in_order, 0)) {

@@ -62,6 +62,7 @@ struct RecordMid {
   bool small_o;            // num_blocks // origin_wave == 0
   bool redo_gflops;        // num_gflops needs origin_gflops_exact (see div_const)
   double num_gflops, total_gb;
+  double log2_origin_max;  // log2(origin_max_occ), see finish_mid
 };
 
 // 2^x for finite x, relative error below 1e-13: split x = n + f with
@@ -111,8 +112,8 @@ struct C100 { static constexpr double value = 100.0; };
 struct C1e9 { static constexpr double value = 1e9; };
 
 // Which occupancy models a kernel instantiation contains.
-//   The lean ones: the origin and every destination of the launch have
-//     OccDevice::lean_ok (the 32-bit NVIDIA-rule model, straight-line) or
+//   The lean ones: every destination's ridge point lies within 2^+-500 and the
+//     origin and every destination of the launch have OccDevice::lean_ok (the 32-bit NVIDIA-rule model, straight-line) or
 //     cdna_lean_ok (the compute-unit model, straight-line), the origin one kind
 //     and the destinations all one kind; nothing else is compiled in and no
 //     branch is uniform over the launch.  kModelLeanGp: NVIDIA-rule devices
@@ -135,6 +136,9 @@ enum : int {
 inline int model_for(const OccDevice& origin, const DestArgs* dests, int n_dest) {
   bool lean = true, gp = true, cdna = true;
   for (int d = 0; d < n_dest; ++d) {
+    // (the lean instantiations also form gamma the shared way, see
+    // roofline_gamma_shared, which wants a ridge point of ordinary magnitude)
+    if (!dests[d].ridge_in_range()) return kModelGeneral;
     lean = lean && dests[d].dev.lean_ok();
     gp = gp && dests[d].dev.lean_gp_ok();
     cdna = cdna && dests[d].dev.cdna_lean_ok();
@@ -243,8 +247,6 @@ struct RecordOut {
   uint8_t status;
 };
 
-// Written with selects rather than branches: the 64 records of a wavefront
-// take all paths between them anyway.
 // log2 of a small-kernel block count (0..63).  PERMUTE: read it from the lane
 // that holds it (needs all 64 lanes of the wavefront active); otherwise gather
 // it from the table in memory.
@@ -278,15 +280,56 @@ __device__ __forceinline__ double roofline_gamma(const DestArgs& p, double num_g
   return (num_gflops < 1e-9 || !metrics) ? 1. : gamma;
 }
 
-template <int MODEL, bool PERMUTE>
-__device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn& r,
-                                               const RecordMid& m, double log2_lane) {
-  RecordOut o;
-  const int32_t regs_d = r.dest_regs >= 0 ? r.dest_regs : r.regs;
-  o.occ_d = occupancy_dev<MODEL, true>(p.dev, r.block, r.smem_total, m.smem, regs_d);
-  o.wave_d = mul_small(p.dev.num_sms, o.occ_d);
+// The same for a launch with several destinations, where the two divisions
+// that do not depend on the destination are made once per record: the
+// intensity I = gflops / gb as the reference forms it (the branch on I > R and
+// the expression below the ridge are then the reference's own arithmetic) and
+// 1 / I = gb / gflops, which gives 0.5 * R / I above the ridge as a product
+// (two roundings instead of one: within 2 ulp).  Needs a ridge point within
+// 2^+-500 (DestArgs::ridge_in_range), so that 1 / I is finite whenever I > R.
+struct Intensity {
+  double value, reciprocal;
+};
 
-  const double gamma = roofline_gamma(p, m.num_gflops, m.total_gb, r.metrics);
+__device__ __forceinline__ Intensity record_intensity(double num_gflops, double total_gb) {
+  return Intensity{num_gflops / total_gb, total_gb / num_gflops};
+}
+
+__device__ __forceinline__ double roofline_gamma_shared(const DestArgs& p, double num_gflops,
+                                                        double total_gb, const Intensity& in,
+                                                        bool metrics) {
+  const bool above = in.value > p.ridge;
+  double gamma = above ? p.half_ridge * in.reciprocal : p.neg_half_over_ridge * in.value + 1.;
+  gamma = (total_gb == 0) ? 0. : gamma;
+  return (num_gflops < 1e-9 || !metrics) ? 1. : gamma;
+}
+
+// log2 of the origin's small-kernel block count, which every destination of a
+// launch uses: looked up once per record.
+template <bool PERMUTE>
+__device__ __forceinline__ void finish_mid(RecordMid& m, double log2_lane) {
+  m.log2_origin_max = log2_count<PERMUTE>(log2_lane, m.origin_max_occ);
+}
+
+// Blocks per multiprocessor on the destination.  It depends on the device only
+// through the occupancy constants, not through num_sms, bandwidth, clock or
+// peak: destinations that agree in those (kSameOccAsPrev) share one evaluation.
+template <int MODEL>
+__device__ __forceinline__ int32_t dest_occupancy(const DestArgs& p, const RecordIn& r,
+                                                  const RecordMid& m) {
+  const int32_t regs_d = r.dest_regs >= 0 ? r.dest_regs : r.regs;
+  return occupancy_dev<MODEL, true>(p.dev, r.block, r.smem_total, m.smem, regs_d);
+}
+
+// Everything after the destination's occupancy.  `gamma` is roofline_gamma or
+// roofline_gamma_shared of the record for this destination; finish_mid has run.
+template <int MODEL, bool PERMUTE>
+__device__ __forceinline__ RecordOut dest_scale(const DestArgs& p, const RecordIn& r,
+                                                const RecordMid& m, int32_t occ_d, double gamma,
+                                                double log2_lane) {
+  RecordOut o;
+  o.occ_d = occ_d;
+  o.wave_d = mul_small(p.dev.num_sms, o.occ_d);
   const bool bad_gamma = !(gamma >= 0 && gamma <= 1);
 
   // `a // wave_o == 0 and a // wave_d == 0`: the second test, and its division
@@ -305,8 +348,8 @@ __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn
   // roofline.py:32-45: (clk_ratio * dest_max_occ / origin_max_occ)^(1-gamma), both
   // counts in 1..63; roofline.py:48-64: bw^gamma * clk^(1-gamma) * sm^(1-gamma)
   const double gamma_compl = 1.0 - gamma;
-  const double log2_small = p.log2_clk + log2_count<PERMUTE>(log2_lane, dest_max_occ) -
-                            log2_count<PERMUTE>(log2_lane, m.origin_max_occ);
+  const double log2_small =
+      p.log2_clk + log2_count<PERMUTE>(log2_lane, dest_max_occ) - m.log2_origin_max;
   // small: (1-gamma) * log2_small; else gamma * L_bw + (1-gamma) * L_clk_sm.  As one
   // expression with selected operands (a zero first term is exact), so that
   // the code stays free of branches.
@@ -324,6 +367,16 @@ __device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn
   o.gamma = gamma;
   o.in_order = status == HBT_ST_OK && !small && fabs(r.t) > 0x1p500;
   return o;
+}
+
+// One record, one destination, start to finish.  Written with selects rather
+// than branches: the 64 records of a wavefront take all paths between them.
+template <int MODEL, bool PERMUTE>
+__device__ __forceinline__ RecordOut dest_part(const DestArgs& p, const RecordIn& r,
+                                               RecordMid& m, double log2_lane) {
+  finish_mid<PERMUTE>(m, log2_lane);
+  const double gamma = roofline_gamma(p, m.num_gflops, m.total_gb, r.metrics);
+  return dest_scale<MODEL, PERMUTE>(p, r, m, dest_occupancy<MODEL>(p, r, m), gamma, log2_lane);
 }
 
 }  // namespace dev

@@ -195,6 +195,43 @@ def test_every_device_pair_with_metrics_mix_and_register_table():
         check(rec, origin, dests, out)
 
 
+def test_destinations_that_share_occupancy_constants():
+    """A launch evaluates the occupancy model once per run of destinations with
+    equal occupancy constants (the library puts equal ones next to each other):
+    every destination's row must still be its own, whatever the order given,
+    and equal what a launch for that destination alone writes."""
+    origin = Device.V100
+    rec, _ = synthetic.kernel_records(30_000, origin, seed=21, metrics_fraction=0.7)
+    rng = np.random.default_rng(21)
+    rec["dest_regs"] = np.where(rng.random(30_000) < 0.3, rng.integers(16, 256, 30_000),
+                                -1).astype(np.int32)
+    kr = KernelRecords.from_numpy(rec)
+    sweep, _ = synthetic.device_sweep(6, seed=1)         # one class: only SMs, bandwidth, clock differ
+    named = [getattr(Device, n) for n in ("T4", "P4000", "RTX2070", "P100", "GTX1080Ti", "P4",
+                                          "RTX2080Ti", "MI355X")]
+    mixed = [named[0], sweep[0], named[1], sweep[1], named[2], named[3], sweep[2], named[4],   # launch 1
+             sweep[3], named[5], named[6], sweep[4], named[7], sweep[5]]                      # launch 2
+    worst = 0.0
+    # a warp size that is no power of two puts the launch on the general instantiation
+    odd = DeviceProperties(name="odd", **dict(Device.V100.as_dict(), warp_size=48))
+    odd2 = DeviceProperties(name="odd2", **dict(Device.V100.as_dict(), warp_size=48, num_sms=33,
+                                                mem_bandwidth_gb=300))
+    for dests in (mixed, sweep, [odd, named[0], odd2, sweep[0], named[2], sweep[1]]):
+        out = wave_scale(kr, origin, dests)
+        check(rec, origin, dests, out)
+        for di, d in enumerate(dests):
+            alone = wave_scale(kr, origin, [d])
+            assert torch.equal(out.occ_dest[di], alone.occ_dest[0]), d.name
+            assert torch.equal(out.wave_dest[di], alone.wave_dest[0]), d.name
+            assert torch.equal(out.status[di], alone.status[0]), d.name
+            a, b = out.time_ns[di].cpu().numpy(), alone.time_ns[0].cpu().numpy()
+            ok = ~np.isnan(b)
+            # gamma above the ridge is a product here and a quotient there: last bits
+            np.testing.assert_allclose(a[ok], b[ok], rtol=1e-13)
+            worst = max(worst, float(np.max(np.abs(a[ok] - b[ok]) / np.abs(b[ok]))))
+    print("several destinations per launch vs one: max relative time difference %.3g" % worst)
+
+
 def test_every_status_and_the_short_circuit(kat):
     base = dict(kat["scaling_record"])
     rows = [
