@@ -11,7 +11,11 @@ inputs resident in HBM.  Prints ONE JSON line:
                 bytes per record / average launch duration (HIP events on the
                 launch stream)
   cpu_baseline  the CPU oracle (C restatement of the reference's per-kernel
-                Python, one thread) on the same records, same machine
+                Python, one thread) on the same records, same machine; under
+                all_cores the same over every host core the box gives this job
+  parity        untimed: the timed launch's outputs against the oracle (integer
+                and status mismatches, largest relative time error), and the
+                MLP against its fp64 evaluation on 4 096 rows
   multi_destination  the same records scaled to the seven other NVIDIA devices of the
                 device table in one launch (records read once)
   large         the same kernel at 64 M records (beyond the 256 MB last-level cache);
@@ -132,6 +136,7 @@ def tile_records(rec, n):
 def mlp_bench(args):
     """configs[2] (and the other kinds of configs[3], one step each): the fused
     MLP at full size, the per-layer path (up to 7168 rows), and a torch CPU baseline."""
+    import numpy as np
     import torch
     from habitat_amd import synthetic
     from habitat_amd.analysis.mlp.mlp import RuntimePredictor
@@ -178,6 +183,22 @@ def mlp_bench(args):
         ys = torch.empty(rows, dtype=torch.float32, device="cuda")
         _, f_launch = time_steps(lambda: rp.predict_batch(xs, out=ys), 200, 50)
         few["rows_%d_us" % rows] = f_launch * 1e3
+    # RuntimePredictor.predict as the reference calls it (mlp.py:252-267): what a
+    # caller waits per call, wall clock, for arguments not asked before (one
+    # hbt_mlp_predict_one: a row through pinned memory, ten launches, a wait) and
+    # for arguments asked before (answered from the predictor's table)
+    n_feat = len(rp.model.features)
+    ops = [list(map(float, x[i, :n_feat])) for i in range(400)]
+    for a_ in ops[:100]:
+        rp.predict(a_, "V100")
+    t0 = time.perf_counter()
+    for a_ in ops[100:]:
+        rp.predict(a_, "V100")
+    few["predict_wall_us"] = (time.perf_counter() - t0) / 300 * 1e6
+    t0 = time.perf_counter()
+    for a_ in ops[100:]:
+        rp.predict(a_, "V100")
+    few["predict_again_wall_us"] = (time.perf_counter() - t0) / 300 * 1e6
     if not args.no_cpu:
         from oracle import mlp as omlp
         sd = rp.model.state_dict()
@@ -186,9 +207,26 @@ def mlp_bench(args):
         for i in range(20):
             omlp.forward_fp32(sd, x[i:i + 1], mu, sigma)
         few["cpu_rows_1_us"] = (time.perf_counter() - t0) / 20 * 1e6
-    few["note"] = ("up to 7168 rows: one launch per layer over the whole GPU "
-                   "(mlp_layer_kernel up to 128 rows, mlp_layer_tile_kernel above); "
-                   "cpu_rows_1_us: torch CPU fp32, batch 1, as the reference predicts")
+        # untimed: the MLP against the fp64 evaluation of the same weights
+        m = min(4096, args.mlp_rows)
+        y64 = omlp.forward_fp64(sd, x[:m], mu, sigma)
+        worst = {}
+        for rows in sorted({1, min(20, m), min(300, m), m}):
+            y = rp.predict_batch(xg[:rows].contiguous()).cpu().numpy().astype("float64")
+            worst["rows_%d" % rows] = float(
+                (abs(y - y64[:rows]) / np.maximum(abs(y64[:rows]), 1e-3)).max())
+        yf = yg[:m].cpu().numpy().astype("float64")      # the timed 1 M-row launch's own output
+        worst["first_%d_of_the_timed_launch" % m] = float(
+            (abs(yf - y64) / np.maximum(abs(y64), 1e-3)).max())
+        mlp["parity"] = {"max_rel_error_vs_fp64": worst, "tolerance": 1e-4,
+                         "floor_on_reference_magnitude": 1e-3,
+                         "against": "oracle/mlp.py forward_fp64 on the first %d rows" % m}
+    few["note"] = ("rows_N_us: GPU time of one forward (HIP events); up to 7168 rows one "
+                   "launch per layer over the whole GPU (mlp_layer_kernel up to 128 rows, "
+                   "mlp_layer_tile_kernel above); predict_wall_us: wall time of one "
+                   "RuntimePredictor.predict call, predict_again_wall_us: of one with arguments "
+                   "asked before; cpu_rows_1_us: torch CPU fp32, batch 1, as the reference "
+                   "predicts")
     mlp["few_rows"] = few
     others = {}
     for other in [k for k in args.mlp_other_kinds.split(",") if k and k != kind]:
@@ -366,6 +404,9 @@ def main():
     # reads the rate a stream of batches would see, the GPU is brought up to
     # its working state with untimed launches first: at least 2 000 untimed
     # launches in all, --warmup of them counted as the warm-up steps.
+    # The same --warmup / --steps protocol without that (the figure a cold,
+    # short run reads; the first call also loads the kernel's code object):
+    cold_wall_ms, cold_launch_ms = time_steps(call, args.steps, args.warmup)
     settle = max(0, 2000 - args.warmup)
     for _ in range(settle):
         call()
@@ -386,11 +427,25 @@ def main():
                    "seed": stats["seed"], "rejected_draws": stats["rejected"]},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
+                     # the same bytes over the wall-clock step (launch overhead of the
+                     # Python loop included): `value` x 68 B / peak
+                     "frac_wall": BYTES_PER_RECORD * rec_per_s / 1e9 / HBM_PEAK_GBS,
+                     # 68 MB fit the 256 MB last-level cache and the same buffers are
+                     # read every step: this point is cache-resident.  The figure
+                     # beyond the cache is copied here from `large` once measured.
+                     "cache_resident": args.records * BYTES_PER_RECORD < 256e6,
+                     "frac_beyond_cache": None,
                      "traffic": TRAFFIC_BYTES_PER_RECORD * args.records,
-                     "traffic_unit": "bytes/launch (FETCH_SIZE + WRITE_SIZE, rocprofv3, "
-                                     "copy-calibrated; see profiles/)",
+                     "traffic_source": "constant from profiles/wave_scale_kernel_1M_and_64M_"
+                                       "records.md (rocprofv3 FETCH_SIZE + WRITE_SIZE per "
+                                       "record, copy-calibrated), not measured in this run",
                      "kernel": "wave_scale_kernel<1, 1, true, unsigned int>", "launch_us": launch_ms * 1e3,
                      "bytes_per_record": BYTES_PER_RECORD},
+        "unsettled": {"ms_per_step": cold_wall_ms, "launch_us": cold_launch_ms * 1e3,
+                      "frac": BYTES_PER_RECORD * args.records / (cold_launch_ms * 1e-3) / 1e9
+                              / HBM_PEAK_GBS,
+                      "what": "the same --warmup/--steps timing made first, before the "
+                              "settle launches (the protocol of the first bench records)"},
     }
 
     def attempt(key, section):
@@ -402,6 +457,29 @@ def main():
             value = {"error": "%s: %s" % (type(exc).__name__, exc)}
         if value is not None:
             result[key] = value
+
+    # ---------------- parity of what was just timed (untimed) ----------------
+    def parity_section():
+        from oracle import lib as olib
+        want = olib.wave_scale(olib.make_device(**origin.as_dict()),
+                               olib.make_device(**dest.as_dict()), rec)
+        torch.cuda.synchronize()
+        t = out.time_ns[0].cpu().numpy()
+        st = out.status[0].cpu().numpy()
+        ok = want["status"] == 0
+        rel = np.abs(t[ok] - want["time_ns"][ok]) / np.abs(want["time_ns"][ok])
+        return {"records": args.records,
+                "occupancy_mismatches": int((out.occ_origin.cpu().numpy() != want["occ_origin"]).sum()
+                                            + (out.occ_dest[0].cpu().numpy() != want["occ_dest"]).sum()),
+                "status_mismatches": int((st != want["status"]).sum()),
+                "non_ok_records": int((~ok).sum()),
+                "nan_where_not_ok": bool(np.all(np.isnan(t[~ok]))),
+                "max_rel_time_error": float(rel.max()) if rel.size else 0.0,
+                "tolerance": 1e-6,
+                "against": "oracle/wave_scaling.c on the same %d records" % args.records}
+
+    if not args.no_cpu:
+        attempt("parity", parity_section)
 
     # ---------------- CPU baseline on the same records ----------------
     def cpu_section():
@@ -415,6 +493,22 @@ def main():
             olib.wave_scale(o, d, rec)
             reps += 1
         c_rate = reps * args.records / (time.perf_counter() - t0)
+        # every core the box gives this job: contiguous slices of the records, one
+        # per thread (the C call releases the interpreter lock)
+        import concurrent.futures
+        cores = max(1, min(int(os.environ.get("OMP_NUM_THREADS", "0")) or os.cpu_count(),
+                           os.cpu_count()))
+        bounds = np.linspace(0, args.records, cores + 1).astype(np.int64)
+        slices = [{k: np.ascontiguousarray(v[a:b]) for k, v in rec.items()}
+                  for a, b in zip(bounds[:-1], bounds[1:])]
+        with concurrent.futures.ThreadPoolExecutor(cores) as pool:
+            one_pass = lambda: list(pool.map(lambda part: olib.wave_scale(o, d, part), slices))
+            one_pass()
+            a_reps, t0 = 0, time.perf_counter()
+            while a_reps < 3 or (time.perf_counter() - t0 < 5.0 and a_reps < 2000):
+                one_pass()
+                a_reps += 1
+            all_rate = a_reps * args.records / (time.perf_counter() - t0)
         m = min(100_000, args.records)
         rows = [{k: v[i].item() for k, v in rec.items()} for i in range(m)]
         t0 = time.perf_counter()
@@ -426,6 +520,10 @@ def main():
             "sample": "oracle/wave_scaling.c (per-record C restatement of the reference's "
                       "Python, libm pow) over the same %d records x %d passes, one thread of %d "
                       "host cores" % (args.records, reps, os.cpu_count()),
+            "all_cores": {
+                "value": all_rate, "unit": "records/s", "cores": cores, "kind": "port",
+                "sample": "the same C restatement on %d threads, one contiguous slice of the "
+                          "%d records each, %d passes" % (cores, args.records, a_reps)},
             "python_per_record": {
                 "value": py_rate, "unit": "records/s", "cores": 1,
                 "sample": "oracle/wave_scaling.py, one Python call chain per record as the "
@@ -521,7 +619,9 @@ def main():
         # launch counts of this section's own: a short run after a cold start
         # reads 60 % high (the kernel instantiation is loaded on first use)
         m_wall, m_launch = time_steps(m_call, 500, 200)
-        per_record = 52 + 17 * len(dests)     # the record is read once per launch
+        # the record is read once and the origin occupancy written once per launch;
+        # per destination: fp64 time + int32 occupancy + status byte
+        per_record = 52 + 4 + 13 * len(dests)
         gbs = per_record * records.n / (m_launch * 1e-3) / 1e9
         return {"destinations": [d.name for d in dests], "launch_us": m_launch * 1e3,
                 "us_per_destination": m_launch * 1e3 / len(dests),
@@ -536,6 +636,9 @@ def main():
     del call, records, out
     if not args.no_large and args.large_records > args.records:
         attempt("large", large_section)
+        if "roofline" in result.get("large", {}):
+            result["roofline"]["frac_beyond_cache"] = result["large"]["roofline"]["frac"]
+            result["roofline"]["records_beyond_cache"] = result["large"]["records"]
         torch.cuda.empty_cache()
         # a size between the two: out of L2, within the last-level cache's reach
         if args.large_records > 16_000_000 > args.records:

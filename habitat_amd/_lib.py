@@ -81,6 +81,7 @@ _SIGNATURES = {
                             C.POINTER(C.c_int)]),
     "hbt_mlp_forward": (C.c_int, [_P, _P, C.c_int64, _P, _P]),
     "hbt_mlp_destroy": (None, [_P]),
+    "hbt_mlp_predict_one": (C.c_int, [_P, _P, C.POINTER(C.c_float), _P]),
     "hbt_mlp_forward_static": (C.c_int, [_P, _P, C.c_int64, _P, _P]),
     "hbt_local_device_spec": (C.c_int, [C.c_int, C.POINTER(DeviceSpec), C.c_char_p, C.c_size_t]),
     "hbt_measure_fp32_fma_gflops": (C.c_int, [C.c_int, C.POINTER(C.c_double)]),

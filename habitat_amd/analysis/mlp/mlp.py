@@ -9,7 +9,9 @@ signature.  The forward pass itself runs in libhabitat_mi.so
 `predict_batch` is the entry that makes it worthwhile.  Training is not part of
 this package.
 """
+import collections
 import ctypes
+import threading
 
 import numpy as np
 import torch
@@ -102,6 +104,20 @@ class _DeviceMLP:
             ctypes.byref(err))
         if not self.handle:
             raise _lib.HabitatLibraryError(err.value, "hbt_mlp_create")
+        # Batches of up to 7168 rows (and what a larger batch leaves over) run
+        # through scratch memory of the handle, so calls on one handle must not
+        # overlap.  Calls that follow each other on one stream never do; a call
+        # on ANOTHER stream than the one before is made to wait for that stream
+        # first, under a lock that also keeps two threads apart.
+        self._lock = threading.Lock()
+        self._last_stream = None
+
+    def _ordered_after_the_call_before(self, stream):
+        """Call with self._lock held."""
+        last = self._last_stream
+        if last is not None and last != stream:
+            stream.wait_stream(last)
+        self._last_stream = stream
 
     def forward(self, raw, out=None, stream=None):
         """raw: [n, in_features] float64 GPU tensor -> [n] float32 GPU tensor."""
@@ -115,12 +131,28 @@ class _DeviceMLP:
             out = torch.empty((n,), dtype=torch.float32, device=raw.device)
         if stream is None:
             stream = torch.cuda.current_stream(raw.device)
-        with torch.cuda.device(raw.device):
+        with self._lock, torch.cuda.device(raw.device):
+            self._ordered_after_the_call_before(stream)
             rc = _lib.lib().hbt_mlp_forward(self.handle, ctypes.c_void_p(raw.data_ptr()), n,
                                             ctypes.c_void_p(out.data_ptr()),
                                             ctypes.c_void_p(stream.cuda_stream))
         _lib.check(rc, "hbt_mlp_forward")
         return out
+
+    def predict_one(self, row):
+        """row: [in_features] float64 numpy array (host) -> float; one
+        hbt_mlp_predict_one call, which waits for the result."""
+        if row.dtype != np.float64 or row.shape != (self.in_features,):
+            raise TypeError("one row of %d float64 features" % self.in_features)
+        out = ctypes.c_float(0.0)
+        stream = torch.cuda.current_stream(self.torch_device)
+        with self._lock, torch.cuda.device(self.torch_device):
+            self._ordered_after_the_call_before(stream)
+            rc = _lib.lib().hbt_mlp_predict_one(self.handle, ctypes.c_void_p(row.ctypes.data),
+                                                ctypes.byref(out),
+                                                ctypes.c_void_p(stream.cuda_stream))
+        _lib.check(rc, "hbt_mlp_predict_one")
+        return out.value
 
     def __del__(self):
         try:
@@ -132,6 +164,12 @@ class _DeviceMLP:
 
 
 class RuntimePredictor:
+    # predictions `predict` remembers: the reference asks for every operation
+    # twice, once with the origin's device features (predictor.py:177-180), and
+    # a trace predicted for one destination after another asks the origin-side
+    # question again each time
+    PREDICT_CACHE_ENTRIES = 4096
+
     def __init__(self, model_name, layers, layer_size, model_path=None):
         self.model_name = model_name
         self.layers = layers
@@ -141,6 +179,7 @@ class RuntimePredictor:
         self.mu = None
         self.sigma = None
         self._gpu = None
+        self._predicted = collections.OrderedDict()
         if model_path is not None:
             self.load_state(model_path)
 
@@ -156,7 +195,7 @@ class RuntimePredictor:
         self.mu = np.asarray(checkpoint["mu"], np.float64)
         self.sigma = np.asarray(checkpoint["sigma"], np.float64)
         self.model.load_state_dict(checkpoint["model"])
-        self._gpu = None
+        self.refresh()
 
     def save_state(self, path):
         torch.save({"mu": self.mu, "sigma": self.sigma, "model": self.model.state_dict()}, path)
@@ -164,11 +203,13 @@ class RuntimePredictor:
     def set_normalization(self, mu, sigma):
         self.mu = np.asarray(mu, np.float64)
         self.sigma = np.asarray(sigma, np.float64)
-        self._gpu = None
+        self.refresh()
 
     def refresh(self):
-        """Re-upload the weights after `self.model` was modified in place."""
+        """Re-upload the weights after `self.model` was modified in place (and
+        forget what `predict` remembered of the old ones)."""
         self._gpu = None
+        self._predicted.clear()
 
     def _device_mlp(self):
         if self._gpu is None:
@@ -180,12 +221,23 @@ class RuntimePredictor:
 
     # -- prediction -----------------------------------------------------------
     def predict(self, kernel_arguments, device_name):
-        """One prediction, as the reference's predict (mlp.py:252-267)."""
+        """One prediction, as the reference's predict (mlp.py:252-267): one C
+        call that waits for the GPU.  Asking again for the same arguments on
+        the same device is answered from a table (cleared by `refresh`)."""
         device_features = get_device_features(device_name, self.device_params)
-        features = np.array(list(kernel_arguments) + device_features, dtype=np.float64)
-        gpu = self._device_mlp()
-        raw = torch.from_numpy(features[None, :]).to(gpu.torch_device)
-        return float(gpu.forward(raw).item())
+        row = list(kernel_arguments) + device_features
+        features = np.array(row, dtype=np.float64)
+        key = features.tobytes()
+        remembered = self._predicted
+        value = remembered.get(key)
+        if value is not None:
+            remembered.move_to_end(key)
+            return value
+        value = self._device_mlp().predict_one(features)
+        remembered[key] = value
+        if len(remembered) > self.PREDICT_CACHE_ENTRIES:
+            remembered.popitem(last=False)
+        return value
 
     def predict_batch(self, raw_features, out=None, stream=None):
         """raw_features: [n, F+4] float64 (numpy array or GPU tensor): operation

@@ -834,6 +834,10 @@ __global__ __launch_bounds__(256) void mlp_last_km_kernel(const LastArgs a) {
                   (part[2][threadIdx.x] + part[3][threadIdx.x])) + a.b_last;
 }
 
+constexpr size_t kOneOutOffset = 512;  // hbt_mlp_predict_one's result within its staging block
+constexpr size_t kOneBytes = 1024;
+static_assert(kMaxInPadded * sizeof(double) <= kOneOutOffset, "a raw row fits below the result");
+
 constexpr int kWaves = 4;  // one wave per SIMD: measured faster than two (fewer, longer MFMA runs between load bursts)
 constexpr size_t kLdsBytes =
     (size_t)(kRows * kStride + (kWaves * 64 / 32) * 32 + kWidth) * sizeof(float);
@@ -855,6 +859,11 @@ struct hbt_mlp {
   const float* w_first_t;  // fc1.weight transposed [kFirstFmaMaxIn][width]; null above that many inputs
   float b_last;
   float* scratch[2];   // per-layer path: two buffers of kScratchFloats activations or partials
+  // hbt_mlp_predict_one: a pinned, device-visible block (one raw row in, one
+  // prediction out at kOneOutOffset) and the lock that serialises its callers
+  unsigned char* one_host;
+  unsigned char* one_device;
+  std::mutex one_lock;
 };
 
 namespace hbt {
@@ -1151,12 +1160,27 @@ hbt_mlp* hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
     return nullptr;
   }
 
-  hbt_mlp* m = new (std::nothrow) hbt_mlp();
-  if (m == nullptr) {
+  void* one_host = nullptr;
+  void* one_device = nullptr;
+  if (hipHostMalloc(&one_host, kOneBytes, hipHostMallocDefault) != hipSuccess ||
+      hipHostGetDevicePointer(&one_device, one_host, 0) != hipSuccess || one_device == nullptr) {
+    (void)hipGetLastError();
+    if (one_host != nullptr) (void)hipHostFree(one_host);
     (void)hipFree(blob);
     *err = HBT_ENOMEM;
     return nullptr;
   }
+  std::memset(one_host, 0, kOneBytes);
+
+  hbt_mlp* m = new (std::nothrow) hbt_mlp();
+  if (m == nullptr) {
+    (void)hipHostFree(one_host);
+    (void)hipFree(blob);
+    *err = HBT_ENOMEM;
+    return nullptr;
+  }
+  m->one_host = static_cast<unsigned char*>(one_host);
+  m->one_device = static_cast<unsigned char*>(one_device);
   unsigned char* base = static_cast<unsigned char*>(blob);
   m->in_features = in_features;
   m->in_padded = in_padded;
@@ -1239,8 +1263,41 @@ int hbt_mlp_forward_static(hbt_mlp* mlp, const double* raw_features, int64_t n, 
   return forward_layers(mlp, raw_features, n, out, buffers, static_cast<hipStream_t>(hip_stream));
 }
 
+int hbt_mlp_predict_one(hbt_mlp* mlp, const double* raw_row, float* out, void* hip_stream) {
+  using namespace hbt;
+  if (mlp == nullptr || raw_row == nullptr || out == nullptr) return HBT_EINVAL;
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    return HBT_EHIP;
+  }
+  if (device != mlp->device) return HBT_EINVAL;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  // the call waits for its stream: a stream under graph capture cannot be used
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+    (void)hipGetLastError();
+    return HBT_EHIP;
+  }
+  if (capture != hipStreamCaptureStatusNone) return HBT_EINVAL;
+
+  std::lock_guard<std::mutex> guard(mlp->one_lock);
+  std::memcpy(mlp->one_host, raw_row, sizeof(double) * (size_t)mlp->in_features);
+  const int rc = forward_layers(mlp, reinterpret_cast<const double*>(mlp->one_device), 1,
+                                reinterpret_cast<float*>(mlp->one_device + kOneOutOffset),
+                                mlp->scratch, stream);
+  if (rc != HBT_OK) return rc;
+  if (hipStreamSynchronize(stream) != hipSuccess) {
+    (void)hipGetLastError();
+    return HBT_EHIP;
+  }
+  std::memcpy(out, mlp->one_host + kOneOutOffset, sizeof(float));
+  return HBT_OK;
+}
+
 void hbt_mlp_destroy(hbt_mlp* mlp) {
   if (mlp == nullptr) return;
+  if (mlp->one_host != nullptr) (void)hipHostFree(mlp->one_host);
   if (mlp->blob != nullptr) (void)hipFree(mlp->blob);
   delete mlp;
 }

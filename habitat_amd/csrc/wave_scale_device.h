@@ -65,6 +65,15 @@ struct RecordMid {
   double log2_origin_max;  // log2(origin_max_occ), see finish_mid
 };
 
+// A double constant held in a scalar register pair.  The compiler would put a
+// 64-bit literal that no instruction can encode into a VECTOR register pair
+// first (two vector moves per use); an FMA reads one scalar operand for free,
+// and the scalar moves that fill it run beside other waves' vector work.
+__device__ __forceinline__ double scalar_const(double c) {
+  asm("" : "+s"(c));
+  return c;
+}
+
 // 2^x for finite x, relative error below 1e-13: split x = n + f with
 // |f| <= 1/2, evaluate e^(f ln 2) by its Taylor polynomial of degree 11
 // ((ln2 / 2)^12 / 12! < 7e-15) and scale by 2^n.
@@ -72,14 +81,14 @@ __device__ __forceinline__ double exp2_poly(double x) {
   const double n = rint(x);
   const double z = (x - n) * 0x1.62e42fefa39efp-1;  // f * ln 2
   double p = 1.0 / 39916800.0;
-  p = fma(p, z, 1.0 / 3628800.0);
-  p = fma(p, z, 1.0 / 362880.0);
-  p = fma(p, z, 1.0 / 40320.0);
-  p = fma(p, z, 1.0 / 5040.0);
-  p = fma(p, z, 1.0 / 720.0);
-  p = fma(p, z, 1.0 / 120.0);
-  p = fma(p, z, 1.0 / 24.0);
-  p = fma(p, z, 1.0 / 6.0);
+  p = fma(p, z, scalar_const(1.0 / 3628800.0));
+  p = fma(p, z, scalar_const(1.0 / 362880.0));
+  p = fma(p, z, scalar_const(1.0 / 40320.0));
+  p = fma(p, z, scalar_const(1.0 / 5040.0));
+  p = fma(p, z, scalar_const(1.0 / 720.0));
+  p = fma(p, z, scalar_const(1.0 / 120.0));
+  p = fma(p, z, scalar_const(1.0 / 24.0));
+  p = fma(p, z, scalar_const(1.0 / 6.0));
   p = fma(p, z, 0.5);
   p = fma(p, z, 1.0);
   p = fma(p, z, 1.0);
@@ -298,8 +307,11 @@ __device__ __forceinline__ Intensity record_intensity(double num_gflops, double 
 __device__ __forceinline__ double roofline_gamma_shared(const DestArgs& p, double num_gflops,
                                                         double total_gb, const Intensity& in,
                                                         bool metrics) {
-  const bool above = in.value > p.ridge;
-  double gamma = above ? p.half_ridge * in.reciprocal : p.neg_half_over_ridge * in.value + 1.;
+  // both expressions are formed and one is selected: no branch, and the
+  // destination's constants are all fetched at the top of its turn
+  const double over = p.half_ridge * in.reciprocal;
+  const double under = p.neg_half_over_ridge * in.value + 1.;
+  double gamma = in.value > p.ridge ? over : under;
   gamma = (total_gb == 0) ? 0. : gamma;
   return (num_gflops < 1e-9 || !metrics) ? 1. : gamma;
 }

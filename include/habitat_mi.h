@@ -278,7 +278,9 @@ int hbt_ratio_scale(const float *pred, int32_t n_dest, int32_t n_rows, const int
  * fp32 as in a torch state_dict; b[] likewise; mu and sigma are the
  * checkpoint's normalisation vectors [in_features] (mlp.py:133-137).  The
  * weights are copied to the current HIP device in the layout the kernels want
- * (this call and hbt_device_table_create are the only ones that allocate).
+ * (this call and hbt_device_table_create are the only ones that allocate
+ * device memory; this one also takes 1 KiB of pinned host memory for
+ * hbt_mlp_predict_one).
  * Returns NULL on failure (and sets *err if err is not NULL).
  */
 typedef struct hbt_mlp hbt_mlp;
@@ -307,6 +309,23 @@ hbt_mlp *hbt_mlp_create(int32_t in_features, int32_t width, int32_t hidden_layer
 int hbt_mlp_forward(hbt_mlp *mlp, const double *raw_features, int64_t n, float *out,
                     void *hip_stream);
 void hbt_mlp_destroy(hbt_mlp *mlp);
+
+/*
+ * One prediction from a row in HOST memory, start to finish: the reference's
+ * RuntimePredictor.predict (analysis/mlp/mlp.py:252-267), which Predictor calls
+ * twice per MLP-predicted operation (analysis/predictor.py:177-180), as one C
+ * call.  raw_row [in_features] and out are HOST memory.  The row goes through
+ * a pinned, device-visible block of the handle (1 KiB, allocated by
+ * hbt_mlp_create), the per-layer kernels of hbt_mlp_forward read it and write
+ * the prediction there, and the call waits for `hip_stream` before it returns:
+ * about 40 us of GPU time, launch-bound.  The result is bit-identical to
+ * hbt_mlp_forward with n = 1.  Uses the handle's scratch like hbt_mlp_forward:
+ * the call must not overlap other calls on the same handle from other streams;
+ * concurrent hbt_mlp_predict_one calls on one handle are serialised inside the
+ * library.  `hip_stream` must not be under graph capture (HBT_EINVAL).  Must be
+ * called with the device of hbt_mlp_create current.
+ */
+int hbt_mlp_predict_one(hbt_mlp *mlp, const double *raw_row, float *out, void *hip_stream);
 
 /*
  * hbt_mlp_forward for callers that cannot allocate device memory or tolerate a

@@ -41,6 +41,12 @@ def check(rec, origin, dests, out, rows=None):
         # atol: a subnormal result (a subnormal measured time, in the adversarial
         # sets) has no 1e-6 relative precision to meet; allow its last bits
         np.testing.assert_allclose(t[ok], want["time_ns"][ok], rtol=TIME_RTOL, atol=1e-320)
+        normal = ok & (np.abs(want["time_ns"]) > 1e-300) & np.isfinite(want["time_ns"])
+        if normal.any():
+            worst = np.max(np.abs(t[normal] - want["time_ns"][normal]) / np.abs(want["time_ns"][normal]))
+            print("wave scaling %s -> %s, %d records: max relative time error vs oracle %.3g "
+                  "(bound %.0e); integers and statuses exact"
+                  % (origin.name, d.name, n, float(worst), TIME_RTOL))
     return n
 
 
