@@ -111,6 +111,9 @@ class _DeviceMLP:
         # first, under a lock that also keeps two threads apart.
         self._lock = threading.Lock()
         self._last_stream = None
+        self._predict_one = _lib.lib().hbt_mlp_predict_one
+        self._one_out = ctypes.c_float(0.0)       # used under self._lock
+        self._one_out_ref = ctypes.byref(self._one_out)
 
     def _ordered_after_the_call_before(self, stream):
         """Call with self._lock held."""
@@ -144,15 +147,25 @@ class _DeviceMLP:
         hbt_mlp_predict_one call, which waits for the result."""
         if row.dtype != np.float64 or row.shape != (self.in_features,):
             raise TypeError("one row of %d float64 features" % self.in_features)
-        out = ctypes.c_float(0.0)
-        stream = torch.cuda.current_stream(self.torch_device)
-        with self._lock, torch.cuda.device(self.torch_device):
-            self._ordered_after_the_call_before(stream)
-            rc = _lib.lib().hbt_mlp_predict_one(self.handle, ctypes.c_void_p(row.ctypes.data),
-                                                ctypes.byref(out),
-                                                ctypes.c_void_p(stream.cuda_stream))
-        _lib.check(rc, "hbt_mlp_predict_one")
-        return out.value
+        out = self._one_out
+        index = self.torch_device.index
+        with self._lock:
+            # (entering torch.cuda.device costs microseconds: only when needed)
+            if torch.cuda.current_device() == index:
+                stream = torch.cuda.current_stream()
+                self._ordered_after_the_call_before(stream)
+                rc = self._predict_one(self.handle, row.ctypes.data, self._one_out_ref,
+                                       stream.cuda_stream)
+            else:
+                with torch.cuda.device(index):
+                    stream = torch.cuda.current_stream()
+                    self._ordered_after_the_call_before(stream)
+                    rc = self._predict_one(self.handle, row.ctypes.data, self._one_out_ref,
+                                           stream.cuda_stream)
+            value = out.value
+        if rc != _lib.HBT_OK:
+            _lib.check(rc, "hbt_mlp_predict_one")
+        return value
 
     def __del__(self):
         try:

@@ -141,23 +141,29 @@ def records_from_kernels(kernels, dest_device, metadata_manager, mode="unified",
     return KernelRecords.from_numpy(rec, device=device or "cuda")
 
 
-_OWN_TIME = operator.attrgetter("_c._run_time_ns")      # this package's MeasuredKernel
-_OWN_BLOCKS = operator.attrgetter("_c._num_blocks")
-_ANY_TIME = operator.attrgetter("run_time_ns")
-_ANY_BLOCKS = operator.attrgetter("num_blocks")
+_LAUNCH_FIELDS = operator.methodcaller("launch_fields")
+_RAW_METRICS = operator.attrgetter("_metrics_kernels")
 
 
 def _fingerprint(passes):
-    """What the cached record columns of `passes` were built from, cheaply:
-    the number of kernels, the sums of their times and block counts, and
-    the passes' own times (about 0.15 ms for 900 kernels, a fraction of what
-    converting and uploading them takes)."""
+    """What the cached record columns of `passes` were built from: every
+    kernel's launch fields and measured time (a hash over the tuples, so a
+    changed block size, register count, shared-memory size, block count or time
+    is seen, and so is a swap of two kernels), how many kernels each pass
+    holds (a kernel moved to a neighbouring pass changes both overheads), the number of raw metric entries
+    behind each kernel (metrics recorded since are seen; a metric already read
+    is cached by the kernel object for good, as in the reference, so its value
+    cannot change under the cache) and the passes' own times.  About 0.3 ms for
+    900 kernels, a fraction of what converting and uploading them takes."""
     kernels = list(itertools.chain.from_iterable(p.kernels for p in passes))
     try:
-        times, blocks = sum(map(_OWN_TIME, kernels)), sum(map(_OWN_BLOCKS, kernels))
+        fields = hash(tuple(map(_LAUNCH_FIELDS, kernels)))
+        metrics = sum(len(m.metrics) for ms in map(_RAW_METRICS, kernels) for m in ms)
     except AttributeError:       # kernel objects of another implementation
-        times, blocks = sum(map(_ANY_TIME, kernels)), sum(map(_ANY_BLOCKS, kernels))
-    return (len(kernels), times, blocks, sum(p.run_time_ms for p in passes))
+        fields = hash(tuple(kernel_fields(k) for k in kernels))
+        metrics = -1
+    return (tuple(len(p.kernels) for p in passes), fields, metrics,
+            sum(p.run_time_ms for p in passes))
 
 
 class Predictor:
@@ -310,9 +316,9 @@ class Predictor:
         return rec, measured_ns, overheads_ns
 
     def clear_record_cache(self):
-        """Forget the cached kernel-record columns (only needed after a change
-        the fingerprint cannot see, such as editing a kernel's metrics or
-        launch configuration in place while its time and block count stay)."""
+        """Forget the cached kernel-record columns (only needed for kernel
+        objects of another implementation whose metrics were changed in place:
+        for those the fingerprint covers launch fields and times only)."""
         self._record_cache.clear()
 
     @staticmethod

@@ -943,13 +943,16 @@ float* static_scratch_of(int device, int* rc) {
 // kernel this path replaced): 512: 156 / 99 / 99; 103.  1280: 263 / 208 / 183;
 // 225.  2560: 382 / 330 / 427; 361.  4096: 506 / 512 / 598; 559.  6144: 744 / 862
 // / 822; 821.
-int tile_k_parts(int m_tiles) {
-  int best = 1, best_cost = (m_tiles + 31) / 32 * 4;  // in quarter steps
-  if (m_tiles <= 128 && (m_tiles + 15) / 16 * 2 < best_cost) {
+int tile_k_parts(int m_tiles, int compute_units) {
+  const int simds = 4 * compute_units;  // 1024 on the GPU the thresholds were measured on
+  // steps a layer takes with K in `ks` parts, in quarters of a whole-K step
+  auto cost = [&](int ks) { return (32 * m_tiles * ks + simds - 1) / simds * (4 / ks); };
+  int best = 1, best_cost = cost(1);
+  if (m_tiles <= simds / 8 && cost(2) < best_cost) {
     best = 2;
-    best_cost = (m_tiles + 15) / 16 * 2;
+    best_cost = cost(2);
   }
-  if (m_tiles <= 64 && (m_tiles + 7) / 8 < best_cost) best = 4;
+  if (m_tiles <= simds / 16 && cost(4) < best_cost) best = 4;
   return best;
 }
 
@@ -973,7 +976,7 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
   l.w_first_t = mlp->w_first_t;
   bool partials = false;
   const float* p_in = nullptr;
-  const int tile_ks = tile_k_parts(m_tiles);
+  const int tile_ks = tile_k_parts(m_tiles, mlp->compute_units);
   for (int layer = 0; layer <= mlp->hidden; ++layer) {
     l.g0 = (layer == 0) ? 0 : mlp->in_padded / 8 + (layer - 1) * (kWidth / 8);
     l.kg = (layer == 0) ? mlp->in_padded / 8 : kWidth / 8;

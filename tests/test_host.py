@@ -366,3 +366,43 @@ def test_feature_extraction_known_answers():
         assert all(type(v) is int for v in got), (kind, label)
         seen.add(kind)
     assert seen == set(classes)
+
+
+def test_record_cache_fingerprint_sees_in_place_changes():
+    """The cached record columns of a pass are reused only while nothing they
+    were built from has changed: any launch field, any time, the order of the
+    kernels, metrics recorded since."""
+    from habitat_amd.analysis.kernels import KernelInstance
+    from habitat_amd.analysis.predictor import _fingerprint
+    trace = synthetic.resnet50_trace(Device.V100, batch=8, seed=3)
+    passes = [rt for op in trace.operations if op.name not in ("conv2d", "linear")
+              for rt in (op.forward, op.backward) if rt is not None][:12]
+    base = _fingerprint(passes)
+    assert _fingerprint(passes) == base
+    k0, k1 = passes[0].kernels[0], passes[3].kernels[0]
+    for field in ("_registers_per_thread", "_block_size", "_static_shared_memory",
+                  "_dynamic_shared_memory", "_num_blocks", "_run_time_ns"):
+        old = getattr(k0._c, field)
+        setattr(k0._c, field, old + 1)
+        assert _fingerprint(passes) != base, field
+        setattr(k0._c, field, old)
+        assert _fingerprint(passes) == base
+    # two kernels exchange their times: every sum stays, the columns do not
+    t0, t1 = k0._c._run_time_ns, k1._c._run_time_ns
+    assert t0 != t1
+    k0._c._run_time_ns, k1._c._run_time_ns = t1, t0
+    assert _fingerprint(passes) != base
+    k0._c._run_time_ns, k1._c._run_time_ns = t0, t1
+    # metrics recorded after the columns were built
+    k0._metrics_kernels.append(KernelInstance("m", 1, 64, 0, 0, 16, 1000, [("dram_read_bytes", 1.0)]))
+    assert _fingerprint(passes) != base
+    k0._metrics_kernels.pop()
+    assert _fingerprint(passes) == base
+    # a kernel moved from one pass to the next one
+    moved = passes[0].kernels.pop()
+    passes[1].kernels.insert(0, moved)
+    assert _fingerprint(passes)[1] == base[1]       # the same kernels in the same order ...
+    assert _fingerprint(passes) != base             # ... but other passes
+    passes[1].kernels.pop(0)
+    passes[0].kernels.append(moved)
+    assert _fingerprint(passes) == base

@@ -85,3 +85,48 @@ def test_static_scratch_forward_rejects_what_it_cannot_hold():
     assert torch.equal(a, rp.predict_batch(raw[:64]))
     assert torch.equal(b, other.predict_batch(raw[:64]))
     assert not torch.equal(a, b)
+
+
+def test_static_scratch_forward_inside_a_hip_graph():
+    """What the entry point is for: a caller under graph capture.  The first
+    call on a device looks the array's address up and is made eagerly; a
+    captured call then replays, with eager work and synchronisations between
+    the replays, to the eager result bit for bit, also after the input rows
+    changed in place."""
+    torch.manual_seed(0)
+    rp = RuntimePredictor("conv2d", 8, 1024)
+    x, mu, sigma = synthetic.mlp_features("conv2d", 600, seed=9)
+    rp.set_normalization(mu, sigma)
+    handle = rp._device_mlp().handle
+    lib = _lib.lib()
+    first, second = torch.from_numpy(x[:300]).cuda(), torch.from_numpy(x[300:]).cuda()
+    raw = first.clone()
+    eager = torch.empty((300,), dtype=torch.float32, device="cuda")
+    assert _forward("hbt_mlp_forward_static", handle, raw, 300, eager) == 0    # outside capture
+    torch.cuda.synchronize()
+    want_first = eager.clone()
+    out = torch.full((300,), -1.0, dtype=torch.float32, device="cuda")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = lib.hbt_mlp_forward_static(handle, ctypes.c_void_p(raw.data_ptr()), 300,
+                                        ctypes.c_void_p(out.data_ptr()),
+                                        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert float(out[0]) == -1.0                      # captured, not run
+    raw.copy_(second)
+    assert _forward("hbt_mlp_forward", handle, raw, 300, eager) == 0
+    torch.cuda.synchronize()
+    want_second = eager.clone()
+    assert not torch.equal(want_first, want_second)
+    for rep in range(4):
+        rows, want = (first, want_first) if rep % 2 == 0 else (second, want_second)
+        raw.copy_(rows)
+        out.fill_(-1.0)
+        graph.replay()
+        # eager work of the program's own between the replays
+        other = rp.predict_batch(first[:40])
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), rep
+        assert torch.equal(other, want_first[:40]) or torch.allclose(other, want_first[:40],
+                                                                     rtol=1e-5, atol=1e-7)
