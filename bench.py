@@ -63,6 +63,9 @@ def parse():
     ap.add_argument("--mlp-kind", default="conv2d")
     ap.add_argument("--mlp-steps", type=int, default=3)
     ap.add_argument("--no-mlp", action="store_true")
+    ap.add_argument("--no-few-rows", action="store_true",
+                    help="skip the MLP timings at 1 to 5911 rows (thousands of launches: "
+                         "leave them out of a counter run on the fused kernel)")
     ap.add_argument("--no-large", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true",
@@ -177,6 +180,8 @@ def mlp_bench(args):
             "sample": "oracle/mlp.py forward_fp32 (torch CPU fp32, one batched forward) on "
                       "the first %d rows, %d torch threads" % (m, threads)}
     # few rows: the reference's own call pattern is one row per call (mlp.py:252-267)
+    if args.no_few_rows:
+        return mlp
     few = {}
     for rows in (1, 48, 108, 512, 1536, 4096, 5911):
         xs = xg[:rows].contiguous()
