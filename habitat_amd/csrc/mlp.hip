@@ -305,18 +305,15 @@ __global__ __launch_bounds__(WAVES * 64, 1) void mlp_fused_kernel(const MlpArgs 
 // The order of every sum is fixed, so results are reproducible.  Same packed
 // weights, same MFMA instruction, same fragment layout as above.
 constexpr int kSplit = 8;            // K-partials per hidden layer, up to kSplitMaxRows rows
-// Rows up to which K is split over workgroups.  Measured per forward at 1 / 8 /
-// 16 / 24 / 32 rows: split 39 44 52 61 71 us (the partials' traffic grows with
-// the rows), whole K 57 us at any of them.
+// Rows up to which K is split over workgroups (the partials' traffic grows with
+// the rows; beyond this the whole-K shapes are faster).
 constexpr int kSplitMaxRows = 20;
-// Largest batch that takes this path (224 m-tiles: 7 steps of the tile kernel).
-// Measured against one round of the fused kernel (940 us whatever it holds up to
-// 8192 rows): 6144 rows 744 us, 7168 rows 862, 7296 rows 975.
+// Largest batch that takes this path: 224 m-tiles, 7 steps of the tile kernel on
+// 256 compute units, just under what one round of the fused kernel costs
+// whatever it holds.  Tuned on 256 compute units.
 constexpr int kLayerMaxRows = 7168;
 // m-tiles up to which the eight-wave shape splits K over two workgroups (128
 // workgroups or fewer per layer would leave half the compute units idle).
-// Measured per forward at 32 / 64 / 128 / 256 rows: 49 52 58 82 us against 57 57
-// 59 65 without; four K-partials were no faster than two.
 constexpr int kHalfKMaxTiles = 4;
 // Input features up to which fc1 of a batch stored by k-group is computed with
 // plain FMAs (mlp_first_fma_kernel); the reference's networks have 8 to 12.
@@ -388,15 +385,7 @@ struct LayerFrag {
 // The instantiations in use: fc1 (FIRST, FINAL, 4 waves) with row-major or
 // k-group output; hidden layers with kSplit K-partials in and out (4 waves,
 // rows masked); hidden layers with two K-partials in and out (8 waves, DEPTH 2,
-// KM).  Until mlp_layer_tile_kernel took over above 128 rows, the eight-wave
-// whole-K shape (FINAL, S_IN 0) ran there; measured for it with KM, us per
-// forward at 256 / 512 / 768 / 1024 / 1536 / 2048 / 4096 rows, as (DEPTH, NT):
-//   (0,1)  67 103 128 161 251 318 588     (0,2) 105 110 160 162 230 298 560
-//   (2,1)  67 103 130 160 274 319 596     (2,2)  95 100 154 154 280 291 605
-//   (4,1)  66 104 130 190 231 325 598     (0,4) 168 172 170 171 310 320 613
-//   (16,1) 71 116 154 194 277 360 693     (2,4) 157 161 158 159 287 299 567
-// (with row-major activations, where a fragment touches 32 cache lines for 32
-// bytes each: 256 rows 74 us, 512 123, 1024 176 with four n-tiles, 4096 637).
+// KM).
 template <bool FIRST, int S_IN, bool FINAL, int WAVES, bool PADDED_ROWS, int DEPTH, int NT = 1,
           bool KM = false, int S_OUT = (FINAL ? 1 : kSplit)>
 __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a) {
@@ -576,25 +565,6 @@ __global__ __launch_bounds__(WAVES * 64) void mlp_layer_kernel(const LayerArgs a
 // tiles per SIMD, rounded up: KS trades a finer rounding (1024 / KS rows per
 // step) against shorter runs per wave.  Activations in and out are stored by
 // k-group (km_index); bias and ReLU are applied on the way out.
-// Measured per forward at 4096 rows with KS = 1: a wave owning 2 x 2 tiles 526
-// us, 1 x 2 tiles 514, one tile 501 (8 ring slots: 503); workgroups numbered
-// m-tile first instead of n-tile first: no difference; two accumulators taking
-// turns (no MFMA waits for the one before it): no difference up to 5120 rows, and
-// above that the 16 registers more cost residency (5911 rows 936 us against 730).
-// Workgroups of 8 or 16
-// waves with K in as many parts (a tile per workgroup, everything summed in
-// LDS) took 57-59 us at 21 to 128 rows, where two workgroups per tile with their
-// K-partials through memory take 49-58: a tile is 3.4 us of ONE compute unit's
-// matrix cores, so few rows want each tile spread over several compute units.
-// fc2 folded into the last hidden layer (every wave leaves its tile's share of
-// the dot product in memory, the wave that completes an m-tile's 32 shares adds
-// them in order; no launch for fc2, no activations written) gained nothing: 512
-// rows 102 us against 99, 4096 rows 511 against 506, 160 rows 60 against 62 -
-// the fc2 launch costs what the count-and-add tail costs (with __threadfence
-// around the count 4096 rows took 591 us: the fences' cache invalidations cost
-// the waves still in their K loop their weights).  A separate fc1 kernel (a
-// workgroup per m-tile standardising the rows once for all n-tiles) was slower
-// below 1024 rows and within 1 % above.
 template <int KS, int SLOTS>
 __global__ __launch_bounds__(256) void mlp_layer_tile_kernel(const LayerArgs a) {
   static_assert(KS == 1 || KS == 2 || KS == 4, "four waves per workgroup");
@@ -691,10 +661,8 @@ __global__ __launch_bounds__(256) void mlp_layer_tile_kernel(const LayerArgs a) 
 // row, this one 8 times), stages its slice of the transposed weights in LDS,
 // and each lane (row m, half h) then produces four consecutive outputs per
 // k-group of the next layer, 1 KiB of contiguous memory per wave and store.
-// Sum order: bias, then k ascending.  Measured against the MFMA kernel: 4096
-// rows 8.4 against 14.1 us, 1536 rows 7.2 against 6.8, 512 rows 5.3 against 4.5
-// (hence kFirstFmaMinTiles); with 2 / 16 / 32 slices instead of 8, 4096 rows take
-// 19.4 / 10.0 / 13.6 us.
+// Sum order: bias, then k ascending.  Faster than the MFMA kernel from about
+// 2048 rows (kFirstFmaMinTiles), slower below.
 __global__ __launch_bounds__(256) void mlp_first_fma_kernel(const LayerArgs a) {
   __shared__ float xs[kRows][kFirstFmaMaxIn + 1];
   __shared__ __attribute__((aligned(16))) float wl[kFirstFmaMaxIn * (kWidth / kFirstFmaSlices)];  // [k][n of the slice]
@@ -838,7 +806,7 @@ constexpr size_t kOneOutOffset = 512;  // hbt_mlp_predict_one's result within it
 constexpr size_t kOneBytes = 1024;
 static_assert(kMaxInPadded * sizeof(double) <= kOneOutOffset, "a raw row fits below the result");
 
-constexpr int kWaves = 4;  // one wave per SIMD: measured faster than two (fewer, longer MFMA runs between load bursts)
+constexpr int kWaves = 4;  // one wave per SIMD: fewer, longer MFMA runs between load bursts than with two
 constexpr size_t kLdsBytes =
     (size_t)(kRows * kStride + (kWaves * 64 / 32) * 32 + kWidth) * sizeof(float);
 
@@ -933,16 +901,13 @@ float* static_scratch_of(int device, int* rc) {
 }
 
 // Into how many parts mlp_layer_tile_kernel splits K for a batch of m_tiles
-// m-tiles.  A layer is 32 m_tiles output tiles on 1024 SIMDs and takes
-// ceil(32 m_tiles KS / 1024) steps of 13.7 / KS us: the finest split is never
-// worse by that count, but a wave's run gets shorter (a run of 32 k-groups is 3.4
-// us, next to about a microsecond until its first fragments arrive) and all
-// workgroups should be resident at once (8 per compute unit), so the coarsest
-// split among the cheapest is taken, KS = 2 up to 4096 rows and KS = 4 up to 2048.
-// Measured per forward, as (rows: us with KS = 1 / 2 / 4; the 8-wave whole-K
-// kernel this path replaced): 512: 156 / 99 / 99; 103.  1280: 263 / 208 / 183;
-// 225.  2560: 382 / 330 / 427; 361.  4096: 506 / 512 / 598; 559.  6144: 744 / 862
-// / 822; 821.
+// m-tiles.  A layer is 32 x m_tiles output tiles on 4 x compute_units SIMDs and
+// takes ceil(32 m_tiles KS / SIMDs) steps of 1 / KS of a whole-K tile's time:
+// the finest split is never worse by that count, but a wave's run gets shorter
+// (a run of 32 k-groups is 3.4 us of MFMAs, next to about a microsecond until
+// its first fragments arrive) and all workgroups should be resident at once (8
+// per compute unit), so the coarsest split among the cheapest is taken: on 256
+// compute units KS = 2 up to 4096 rows and KS = 4 up to 2048.
 int tile_k_parts(int m_tiles, int compute_units) {
   const int simds = 4 * compute_units;  // 1024 on the GPU the thresholds were measured on
   // steps a layer takes with K in `ks` parts, in quarters of a whole-K step

@@ -15,9 +15,7 @@ constexpr int kMaxDestPerLaunch = 8;
 // Consecutive records one thread of the kernel's main instantiation owns: each
 // of its column accesses is one load or store of this many elements, and the
 // columns must be aligned to that many elements (otherwise the one-record
-// instantiation runs).  Measured under continuous launches, with the
-// workgroup size that suits each best: one record per thread 11.7 us at 1 M
-// records and 687 us at 64 M, two 11.8 and 725, four 15.0 and 800.
+// instantiation runs).  One is fastest at every size tried.
 constexpr int kVectorRecords = 1;
 
 // Everything about one (origin, destination) pair that does not depend on the

@@ -8,8 +8,8 @@
 // and the scaled time.
 //
 // Data layout: structure of arrays, one column per record field.  A thread owns
-// kVectorRecords consecutive records (one, as measured best; the code is written
-// for any number), so a wavefront reads 256 contiguous bytes of every int32
+// kVectorRecords consecutive records (one; the code is written for any
+// number), so a wavefront reads 256 contiguous bytes of every int32
 // column and 512 of every fp64 column; stores likewise.  All loads of a
 // thread are issued before any arithmetic and all stores after it, so that no
 // wait for a load also waits for a store.  Device constants travel in the
@@ -36,19 +36,9 @@ namespace {
 using namespace dev;
 
 constexpr int kRecPerThread = kVectorRecords;
-// Two wavefronts per workgroup.  Measured under continuous launches with one
-// record per thread: 128 threads 11.7 us at 1 M records and 687 us at 64 M,
-// 64 threads 11.6 and 719, 256 threads 12.2 and 709.  (With two records per
-// thread: 64 threads 11.7 us, 128 11.9, 256 12.5, 512 13.5, and 512 was the only
-// size that ran faster, 12.3 us, for the first milliseconds after idle.)
+// Two wavefronts per workgroup: fresh short waves taking consecutive 128-record
+// chunks keep the chip on one contiguous window of every column.
 constexpr int kBlock = 128;
-// Tried and dropped: a smaller grid whose waves walk over the batch in strides of
-// the whole grid and issue the loads of their next 64 records before computing
-// on the ones they hold (74 VGPRs, 6 waves per SIMD).  1 M records: 11.8 us with
-// 5209 workgroups (1.5 turns per wave), 12.5-13.7 with 2605-3907, 15.1 with 1563,
-// against 11.3; 64 M records 890-960 us against 696.  Fresh short waves taking
-// consecutive chunks keep the chip on one contiguous window of every column;
-// waves that come back for chunks a whole grid further on do not.
 
 // N consecutive elements as one register group (a scalar when N is 1).
 template <class T, int N>
@@ -75,8 +65,7 @@ __device__ __forceinline__ void vec_set(typename VecOf<T, N>::type& v, int k, T 
 //
 // Every column is read once and every output written once, so both directions
 // carry the non-temporal hint: the lines are not kept in L2 or the last-level
-// cache at the expense of each other.  Measured against plain accesses:
-// 745 vs 825 us at 64 M records, 13.0 vs 13.8 us at 1 M.
+// cache at the expense of each other.
 template <class T, int R, class Index>
 __device__ __forceinline__ void load_r(const T* __restrict__ p, Index i, T (&out)[R]) {
   using V = typename VecOf<T, R>::type;
