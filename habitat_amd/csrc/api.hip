@@ -38,7 +38,7 @@ DestArgs make_dest_args(const hbt_device_spec& o, const hbt_device_spec& d) {
   return p;
 }
 
-static bool same_occupancy_constants(OccDevice a, OccDevice b) {
+bool same_occupancy_constants(OccDevice a, OccDevice b) {
   a.num_sms = b.num_sms = 0;
   a.flags &= ~kSameOccAsPrev;
   b.flags &= ~kSameOccAsPrev;

@@ -17,6 +17,7 @@
 // column kernel runs.
 #include <hip/hip_runtime.h>
 
+#include <chrono>
 #include <cstdint>
 #include <cstring>
 #include <mutex>
@@ -47,6 +48,10 @@ struct HostRecordArgs {
   int32_t* occ_origin;
   int32_t* occ_dest;
   uint8_t* status;
+  // a launch of ONE workgroup stores done_value here (host-visible memory) once
+  // its results are in place, so that the caller need not wait for the stream
+  uint32_t* done_flag;  // nullable
+  uint32_t done_value;
   OriginArgs origin;
   DestArgs dest;
 };
@@ -58,34 +63,41 @@ using f64x2 = double __attribute__((ext_vector_type(2)));
 template <int MODEL>
 __global__ __launch_bounds__(kBlock) void wave_scale_records_kernel(const HostRecordArgs a) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i >= a.n) return;
-  const char* p = reinterpret_cast<const char*>(a.rec + i);
-  const i32x4 q0 = *reinterpret_cast<const i32x4*>(p);
-  const i32x4 q1 = *reinterpret_cast<const i32x4*>(p + 16);
-  const f64x2 d0 = *reinterpret_cast<const f64x2*>(p + 32);
-  const f64x2 d1 = *reinterpret_cast<const f64x2*>(p + 48);
-  RecordIn r;
-  r.nb = q0[0];
-  r.block = q0[1];
-  r.smem_total = smem_sum(q0[3], q0[2]);
-  r.regs = q1[0];
-  r.dest_regs = q1[1];
-  r.metrics = q1[2] != 0;
-  r.t = d0[0];
-  r.eff = d0[1];
-  r.rd = d1[0];
-  r.wr = d1[1];
+  if (i < a.n) {
+    const char* p = reinterpret_cast<const char*>(a.rec + i);
+    const i32x4 q0 = *reinterpret_cast<const i32x4*>(p);
+    const i32x4 q1 = *reinterpret_cast<const i32x4*>(p + 16);
+    const f64x2 d0 = *reinterpret_cast<const f64x2*>(p + 32);
+    const f64x2 d1 = *reinterpret_cast<const f64x2*>(p + 48);
+    RecordIn r;
+    r.nb = q0[0];
+    r.block = q0[1];
+    r.smem_total = smem_sum(q0[3], q0[2]);
+    r.regs = q1[0];
+    r.dest_regs = q1[1];
+    r.metrics = q1[2] != 0;
+    r.t = d0[0];
+    r.eff = d0[1];
+    r.rd = d1[0];
+    r.wr = d1[1];
 
-  RecordMid m = origin_part<MODEL>(a.origin, r);
-  if (__builtin_expect(m.redo_gflops, 0))
-    m.num_gflops = origin_gflops_exact(a.origin.peak_gflops, r.eff, r.t);
-  RecordOut o = dest_part<MODEL, false>(a.dest, r, m, 0.0);
-  if (__builtin_expect(o.in_order, 0))
-    o.t = scaled_time_in_order(r.t, o.gamma, a.dest.log2_bw, a.dest.log2_clk, a.dest.log2_clk_sm);
-  a.time_ns[i] = o.t;
-  a.occ_origin[i] = m.occ_o;
-  a.occ_dest[i] = o.occ_d;
-  a.status[i] = o.status;
+    RecordMid m = origin_part<MODEL>(a.origin, r);
+    if (__builtin_expect(m.redo_gflops, 0))
+      m.num_gflops = origin_gflops_exact(a.origin.peak_gflops, r.eff, r.t);
+    RecordOut o = dest_part<MODEL, false>(a.dest, r, m, 0.0);
+    if (__builtin_expect(o.in_order, 0))
+      o.t = scaled_time_in_order(r.t, o.gamma, a.dest.log2_bw, a.dest.log2_clk, a.dest.log2_clk_sm);
+    a.time_ns[i] = o.t;
+    a.occ_origin[i] = m.occ_o;
+    a.occ_dest[i] = o.occ_d;
+    a.status[i] = o.status;
+  }
+  if (a.done_flag != nullptr) {       // uniform; the launch is one workgroup
+    __threadfence_system();           // this thread's results, then ...
+    __syncthreads();                  // ... everybody's
+    if (threadIdx.x == 0)
+      __hip_atomic_store(a.done_flag, a.done_value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
 }
 
 // The staging block of one GPU: kChunk records in, their results out.
@@ -93,12 +105,14 @@ struct Staging {
   std::mutex lock;  // one call at a time per device: the block is shared
   unsigned char* host = nullptr;
   unsigned char* device = nullptr;
+  uint32_t calls = 0;  // numbers the one-workgroup launches: the value they publish
 };
 constexpr size_t kOffTime = (size_t)kChunk * sizeof(hbt_kernel_record);
 constexpr size_t kOffOccOrigin = kOffTime + (size_t)kChunk * sizeof(double);
 constexpr size_t kOffOccDest = kOffOccOrigin + (size_t)kChunk * sizeof(int32_t);
 constexpr size_t kOffStatus = kOffOccDest + (size_t)kChunk * sizeof(int32_t);
-constexpr size_t kStagingBytes = kOffStatus + (size_t)kChunk;
+constexpr size_t kOffDone = kOffStatus + (size_t)kChunk;
+constexpr size_t kStagingBytes = kOffDone + 64;
 constexpr int kMaxDevices = 64;
 Staging g_staging[kMaxDevices];
 
@@ -114,6 +128,7 @@ int staging_ready(Staging& st) {
   }
   st.host = static_cast<unsigned char*>(h);
   st.device = static_cast<unsigned char*>(d);
+  std::memset(st.host + kOffDone, 0, 64);
   return HBT_OK;
 }
 
@@ -136,6 +151,17 @@ int stream_usable(hipStream_t stream, int device) {
 }
 
 }  // namespace
+
+bool wait_published(const uint32_t* flag, uint32_t value) {
+  using clock = std::chrono::steady_clock;
+  const clock::time_point give_up = clock::now() + std::chrono::microseconds(200);
+  for (;;) {
+    for (int spin = 0; spin < 64; ++spin)
+      if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) == value) return true;
+    if (clock::now() > give_up) return false;
+  }
+}
+
 }  // namespace hbt
 
 extern "C" {
@@ -179,12 +205,19 @@ int hbt_wave_scale_host_records(const hbt_device_spec* origin, const hbt_device_
     std::memcpy(st.host, records + done, (size_t)m * sizeof(hbt_kernel_record));
     a.n = m;
     const dim3 grid((unsigned)((m + kBlock - 1) / kBlock));
+    // one workgroup (one kernel, a pass of a few kernels): it publishes its own
+    // completion, see wait_published
+    const bool publishes = grid.x == 1;
+    a.done_flag = publishes ? reinterpret_cast<uint32_t*>(st.device + kOffDone) : nullptr;
+    a.done_value = publishes ? ++st.calls : 0;
     dev::with_model(model, [&](auto mc) {
       hipLaunchKernelGGL(wave_scale_records_kernel<decltype(mc)::value>, grid, dim3(kBlock), 0,
                          stream, a);
     });
     if (hipGetLastError() != hipSuccess) return HBT_EHIP;
-    if (hipStreamSynchronize(stream) != hipSuccess) {
+    if (!(publishes &&
+          wait_published(reinterpret_cast<const uint32_t*>(st.host + kOffDone), a.done_value)) &&
+        hipStreamSynchronize(stream) != hipSuccess) {
       (void)hipGetLastError();
       return HBT_EHIP;
     }

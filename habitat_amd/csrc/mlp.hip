@@ -37,6 +37,7 @@
 #include <vector>
 
 #include "../../include/habitat_mi.h"
+#include "wave_scale.h"
 
 namespace hbt {
 
@@ -713,7 +714,17 @@ struct LastArgs {
   int64_t n;
   int32_t m_pad;
   float* out;            // [n]
+  // hbt_mlp_predict_one: once out[0] is written, done_value is stored here
+  // (host-visible memory) so that the caller need not wait for the stream
+  uint32_t* done_flag;   // nullable
+  uint32_t done_value;
 };
+
+// Publishes `value` to a waiting host thread after this thread's earlier stores.
+__device__ __forceinline__ void publish_done(uint32_t* flag, uint32_t value) {
+  __threadfence_system();
+  __hip_atomic_store(flag, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 // fc2 after the per-layer kernels: one wavefront per row.  S_IN as in mlp_layer_kernel.
 template <int S_IN>
@@ -747,7 +758,10 @@ __global__ __launch_bounds__(256) void mlp_last_kernel(const LastArgs a) {
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off);
-  if (lane == 0) a.out[row] = sum + a.b_last;
+  if (lane == 0) {
+    a.out[row] = sum + a.b_last;
+    if (a.done_flag != nullptr && row == 0) publish_done(a.done_flag, a.done_value);
+  }
 }
 
 // fc2 from activations stored by k-group: one workgroup per m-tile, its four
@@ -802,7 +816,8 @@ __global__ __launch_bounds__(256) void mlp_last_km_kernel(const LastArgs a) {
                   (part[2][threadIdx.x] + part[3][threadIdx.x])) + a.b_last;
 }
 
-constexpr size_t kOneOutOffset = 512;  // hbt_mlp_predict_one's result within its staging block
+constexpr size_t kOneOutOffset = 512;   // hbt_mlp_predict_one's result within its staging block
+constexpr size_t kOneDoneOffset = 768;  // and the call number the last kernel publishes after it
 constexpr size_t kOneBytes = 1024;
 static_assert(kMaxInPadded * sizeof(double) <= kOneOutOffset, "a raw row fits below the result");
 
@@ -831,6 +846,7 @@ struct hbt_mlp {
   // prediction out at kOneOutOffset) and the lock that serialises its callers
   unsigned char* one_host;
   unsigned char* one_device;
+  uint32_t one_calls;      // numbers the calls: the value the kernel publishes
   std::mutex one_lock;
 };
 
@@ -925,7 +941,8 @@ int tile_k_parts(int m_tiles, int compute_units) {
 // activations or K-partials (each at least max(n rounded up to 32, kSplit * 32)
 // x kWidth floats): the handle's, or the library's static ones.
 int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* out,
-                   float* const buffers[2], hipStream_t stream) {
+                   float* const buffers[2], hipStream_t stream, uint32_t* done_flag = nullptr,
+                   uint32_t done_value = 0) {
   using namespace hbt;
   const int m_tiles = (int)((n + kRows - 1) / kRows);
   const bool split_k = n <= kSplitMaxRows;
@@ -989,6 +1006,8 @@ int forward_layers(hbt_mlp* mlp, const double* raw_features, int64_t n, float* o
   z.bias_in = mlp->bias + (size_t)mlp->hidden * kWidth;
   z.w_last = mlp->w_last; z.b_last = mlp->b_last;
   z.n = n; z.m_pad = l.m_pad; z.out = out;
+  z.done_flag = split_k ? done_flag : nullptr;  // (only the few-row shape publishes)
+  z.done_value = done_value;
   const dim3 rows_grid((unsigned)((n + 3) / 4));
   if (partials && split_k)
     hipLaunchKernelGGL(mlp_last_kernel<kSplit>, rows_grid, dim3(256), 0, stream, z);
@@ -1251,11 +1270,18 @@ int hbt_mlp_predict_one(hbt_mlp* mlp, const double* raw_row, float* out, void* h
 
   std::lock_guard<std::mutex> guard(mlp->one_lock);
   std::memcpy(mlp->one_host, raw_row, sizeof(double) * (size_t)mlp->in_features);
+  const uint32_t call = ++mlp->one_calls;
   const int rc = forward_layers(mlp, reinterpret_cast<const double*>(mlp->one_device), 1,
                                 reinterpret_cast<float*>(mlp->one_device + kOneOutOffset),
-                                mlp->scratch, stream);
+                                mlp->scratch, stream,
+                                reinterpret_cast<uint32_t*>(mlp->one_device + kOneDoneOffset), call);
   if (rc != HBT_OK) return rc;
-  if (hipStreamSynchronize(stream) != hipSuccess) {
+  // The last kernel publishes the call's number once the prediction is in the
+  // block: watching for it takes microseconds less than waiting for the
+  // stream's completion signal.  Should it not show up in time, the stream is
+  // waited for, which is always right.
+  if (!hbt::wait_published(reinterpret_cast<const uint32_t*>(mlp->one_host + kOneDoneOffset), call) &&
+      hipStreamSynchronize(stream) != hipSuccess) {
     (void)hipGetLastError();
     return HBT_EHIP;
   }

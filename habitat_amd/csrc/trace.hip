@@ -17,8 +17,8 @@
 //                        per-destination sum of those and the number replaced.
 //
 // Destinations live in a device-resident table (hbt_device_table) so that one
-// launch covers all of them: blockIdx.y is the destination, and its constants
-// come through scalar loads.
+// launch covers all of them: blockIdx.y is a group of destinations, and their
+// constants come through scalar loads.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -48,10 +48,16 @@ namespace {
 using namespace dev;
 
 constexpr int kBlock = 256;
+// Destinations one thread of wave_scale_sum_kernel walks over (blockIdx.y counts
+// groups of this many): the record is loaded and its origin part computed once
+// per group, and the occupancy model runs once per run of destinations with
+// equal occupancy constants within the group.
+constexpr int kSumGroup = 8;
 
 struct SumArgs {
   int64_t n;
   int32_t n_segments;
+  int32_t n_dest;
   const int32_t* num_blocks;
   const int32_t* block_size;
   const int32_t* dynamic_smem;
@@ -76,13 +82,14 @@ __global__ void fill_zero_kernel(double* sums, int64_t n_sums, int32_t* bad, int
   if (bad != nullptr && i < n_bad) bad[i] = 0;
 }
 
-// One thread per (record, destination).  Within a wavefront, consecutive
-// records of the same segment are summed with a segmented scan and the last
-// lane of each run adds the run's total to the segment's sum.
+// One thread per record and group of kSumGroup destinations.  Within a
+// wavefront, consecutive records of the same segment are summed with a
+// segmented scan and the last lane of each run adds the run's total to the
+// segment's sum, per destination.
 template <int MODEL>
 __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a) {
-  const int d = blockIdx.y;
-  const DestArgs& p = a.dests[d];
+  const int d0 = blockIdx.y * kSumGroup;
+  const int d1 = d0 + kSumGroup < a.n_dest ? d0 + kSumGroup : a.n_dest;
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   const int lane = threadIdx.x & 63;
   const bool in_range = i < a.n;
@@ -105,16 +112,7 @@ __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a)
   RecordMid m = origin_part<MODEL>(a.origin, r);
   if (__builtin_expect(m.redo_gflops, 0))
     m.num_gflops = origin_gflops_exact(a.origin.peak_gflops, r.eff, r.t);
-  RecordOut o = dest_part<MODEL, false>(p, r, m, 0.0);
-  if (__builtin_expect(o.in_order, 0))
-    o.t = scaled_time_in_order(r.t, o.gamma, p.log2_bw, p.log2_clk, p.log2_clk_sm);
-
-  const bool ok = in_range && o.status == HBT_ST_OK;
-  double v = ok ? o.t : 0.0;
-  if (a.out_bad != nullptr) {
-    const unsigned long long bad = __ballot(in_range && o.status != HBT_ST_OK);
-    if (lane == 0 && bad != 0) atomicAdd(a.out_bad + d, (int32_t)__popcll(bad));
-  }
+  finish_mid<false>(m, 0.0);
 
   // Runs of equal segment ids get increasing run numbers, so that equal run
   // numbers at any distance mean "same run" even if a segment id repeats later.
@@ -122,16 +120,34 @@ __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a)
   const bool head = lane == 0 || prev_seg != seg;
   const unsigned long long heads = __ballot(head);
   const int32_t run = (int32_t)__popcll(heads & ((2ull << lane) - 1ull));
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const double other = __shfl_up(v, off);
-    const int32_t other_run = __shfl_up(run, off);
-    if (lane >= off && other_run == run) v += other;
-  }
   const int32_t next_run = __shfl_down(run, 1);
   const bool tail = lane == 63 || next_run != run;
-  if (tail && in_range && seg >= 0 && seg < a.n_segments)
-    unsafeAtomicAdd(a.out_sum + (int64_t)d * a.n_segments + seg, v);
+  const bool adds = tail && in_range && seg >= 0 && seg < a.n_segments;
+
+  int32_t occ_d = 0;
+  for (int d = d0; d < d1; ++d) {
+    const DestArgs& p = a.dests[d];
+    // the first destination of a group never carries the mark
+    if (!(p.dev.flags & kSameOccAsPrev)) occ_d = dest_occupancy<MODEL>(p, r, m);
+    const double gamma = roofline_gamma(p, m.num_gflops, m.total_gb, r.metrics);
+    RecordOut o = dest_scale<MODEL, false>(p, r, m, occ_d, gamma, 0.0);
+    if (__builtin_expect(o.in_order, 0))
+      o.t = scaled_time_in_order(r.t, o.gamma, p.log2_bw, p.log2_clk, p.log2_clk_sm);
+
+    const bool ok = in_range && o.status == HBT_ST_OK;
+    double v = ok ? o.t : 0.0;
+    if (a.out_bad != nullptr) {
+      const unsigned long long bad = __ballot(in_range && o.status != HBT_ST_OK);
+      if (lane == 0 && bad != 0) atomicAdd(a.out_bad + d, (int32_t)__popcll(bad));
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const double other = __shfl_up(v, off);
+      const int32_t other_run = __shfl_up(run, off);
+      if (lane >= off && other_run == run) v += other;
+    }
+    if (adds) unsafeAtomicAdd(a.out_sum + (int64_t)d * a.n_segments + seg, v);
+  }
 }
 
 struct GammaArgs {
@@ -258,7 +274,13 @@ hbt_device_table* hbt_device_table_create(const hbt_device_spec* origin,
   t->device = device;
   t->origin = make_origin_args(*origin);
   std::vector<DestArgs> host((size_t)n_dest);
-  for (int32_t d = 0; d < n_dest; ++d) host[d] = make_dest_args(*origin, dests[d]);
+  for (int32_t d = 0; d < n_dest; ++d) {
+    host[d] = make_dest_args(*origin, dests[d]);
+    // within a group of kSumGroup destinations, one that has the occupancy
+    // constants of the one before it shares that one's occupancies
+    if (d % kSumGroup != 0 && same_occupancy_constants(host[d - 1].dev, host[d].dev))
+      host[d].dev.flags |= kSameOccAsPrev;
+  }
   t->model = dev::model_for(t->origin.dev, host.data(), n_dest);
   t->dests = nullptr;
   const size_t bytes = sizeof(DestArgs) * (size_t)n_dest;
@@ -322,6 +344,7 @@ int hbt_wave_scale_sum(const hbt_device_table* table, int64_t n, const int32_t* 
   SumArgs a{};
   a.n = n;
   a.n_segments = n_segments;
+  a.n_dest = table->n_dest;
   a.num_blocks = num_blocks; a.block_size = block_size; a.dynamic_smem = dynamic_smem;
   a.static_smem = static_smem; a.regs = regs; a.dest_regs = dest_regs;
   a.run_time_ns = run_time_ns; a.flop_sp_efficiency = flop_sp_efficiency;
@@ -330,7 +353,7 @@ int hbt_wave_scale_sum(const hbt_device_table* table, int64_t n, const int32_t* 
   a.out_sum = out_sum; a.out_bad = out_bad;
   a.dests = table->dests;
   a.origin = table->origin;
-  const dim3 grid((unsigned)blocks, (unsigned)table->n_dest);
+  const dim3 grid((unsigned)blocks, (unsigned)((table->n_dest + kSumGroup - 1) / kSumGroup));
   dev::with_model(table->model, [&](auto m) {
     hipLaunchKernelGGL(wave_scale_sum_kernel<decltype(m)::value>, grid, dim3(kBlock), 0, stream, a);
   });

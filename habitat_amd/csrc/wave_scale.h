@@ -41,6 +41,9 @@ struct DestArgs {
 // caller's index of the destination now at position i.
 void group_by_occupancy(DestArgs* dests, int32_t* order, int n);
 
+// Everything in the two but num_sms (and the kSameOccAsPrev mark) is equal.
+bool same_occupancy_constants(OccDevice a, OccDevice b);
+
 // The origin device's share of the constants.
 struct OriginArgs {
   OccDevice dev;
@@ -82,6 +85,12 @@ struct WaveScaleArgs {
 
 OriginArgs make_origin_args(const hbt_device_spec& origin);
 DestArgs make_dest_args(const hbt_device_spec& origin, const hbt_device_spec& dest);
+
+// Host side of a kernel that publishes `value` in host-visible memory when its
+// results are in place (a system-scope release store after them): watches
+// `flag` for up to about 200 microseconds.  False when the value did not show
+// up; the caller then waits for the stream instead.
+bool wait_published(const uint32_t* flag, uint32_t value);
 
 // `vectorised` needs every column, and every destination's row of the outputs,
 // aligned to kVectorRecords elements of its type.
