@@ -86,61 +86,10 @@ __device__ __forceinline__ void store_r(T* __restrict__ p, Index i, const T (&in
   __builtin_nontemporal_store(v, reinterpret_cast<V*>(reinterpret_cast<char*>(p) + (size_t)byte));
 }
 
-// An output column as a buffer resource (32-bit offsets only): a store then
-// takes the column's base from scalar registers and the lane's byte offset as
-// one 32-bit register, with no 64-bit address arithmetic, and a column the
-// caller left out (null) becomes an empty buffer, whose stores the hardware
-// drops: no branch around them.
-using u32x2 = unsigned int __attribute__((ext_vector_type(2)));
-using u32x4 = unsigned int __attribute__((ext_vector_type(4)));
-
-template <class T>
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t out_column(T* p, uint32_t n) {
-  return __builtin_amdgcn_make_buffer_rsrc(p, 0, p != nullptr ? (int)(n * (uint32_t)sizeof(T)) : 0,
-                                           0x00020000);
-}
-
-// R consecutive elements of such a column starting at element i (non-temporal,
-// like store_r).
-template <class T, int R>
-__device__ __forceinline__ void store_column(__amdgpu_buffer_rsrc_t column, uint32_t i,
-                                             const T (&in)[R]) {
-  static_assert(sizeof(T) * R <= 16, "one store instruction");
-  constexpr int kNonTemporal = 2;
-  const int byte = (int)(i * (uint32_t)sizeof(T));
-  unsigned char raw[sizeof(T) * R];
-  __builtin_memcpy(raw, in, sizeof(raw));
-  if constexpr (sizeof(raw) == 1) {
-    __builtin_amdgcn_raw_buffer_store_b8(raw[0], column, byte, 0, kNonTemporal);
-  } else if constexpr (sizeof(raw) == 2) {
-    unsigned short v;
-    __builtin_memcpy(&v, raw, 2);
-    __builtin_amdgcn_raw_buffer_store_b16(v, column, byte, 0, kNonTemporal);
-  } else if constexpr (sizeof(raw) == 4) {
-    unsigned int v;
-    __builtin_memcpy(&v, raw, 4);
-    __builtin_amdgcn_raw_buffer_store_b32(v, column, byte, 0, kNonTemporal);
-  } else if constexpr (sizeof(raw) == 8) {
-    u32x2 v;
-    __builtin_memcpy(&v, raw, 8);
-    __builtin_amdgcn_raw_buffer_store_b64(v, column, byte, 0, kNonTemporal);
-  } else {
-    static_assert(sizeof(raw) == 16, "1, 2, 4, 8 or 16 bytes");
-    u32x4 v;
-    __builtin_memcpy(&v, raw, 16);
-    __builtin_amdgcn_raw_buffer_store_b128(v, column, byte, 0, kNonTemporal);
-  }
-}
-
-// An optional output column: through a buffer resource when the launch has
-// 32-bit offsets, else a global store behind a test for null.
+// An optional output column (null = the caller does not want it).
 template <class T, int R, class Index>
-__device__ __forceinline__ void store_out(T* p, Index n, Index i, const T (&in)[R]) {
-  if constexpr (sizeof(Index) == 4 && sizeof(T) * R <= 16) {
-    store_column<T, R>(out_column(p, n), i, in);
-  } else {
-    if (p != nullptr) store_r<T, R>(p, i, in);
-  }
+__device__ __forceinline__ void store_out(T* __restrict__ p, Index i, const T (&in)[R]) {
+  if (p != nullptr) store_r<T, R>(p, i, in);
 }
 
 // Records i .. i+R-1 (all below n) for every destination of the launch.
@@ -238,11 +187,10 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
       in_order = in_order || o.in_order;
     }
     const DestOut& w = a.out[d];
-    const Index n = (Index)a.n;
-    store_out<double, R>(w.time_ns, n, i, ot);
-    store_out<int32_t, R>(w.occ, n, i, occ_d);
-    store_out<int32_t, R>(w.wave, n, i, wave_d);
-    store_out<uint8_t, R>(w.status, n, i, st);
+    store_r<double, R>(w.time_ns, i, ot);
+    store_out<int32_t, R>(w.occ, i, occ_d);
+    store_out<int32_t, R>(w.wave, i, wave_d);
+    store_out<uint8_t, R>(w.status, i, st);
     // Run times beyond 2^+-500 ns (see dest_scale): the time is formed again in
     // the reference's order of operations and stored over the first one, after
     // everything else, where the rare call costs the other records nothing.
@@ -262,8 +210,8 @@ __device__ __forceinline__ void process(const WaveScaleArgs& a, Index i) {
     int32_t occ_o[R], wave_o[R];
 #pragma unroll
     for (int k = 0; k < R; ++k) { occ_o[k] = mid[k].occ_o; wave_o[k] = mid[k].wave_o; }
-    store_out<int32_t, R>(a.out_occ_origin, (Index)a.n, i, occ_o);
-    store_out<int32_t, R>(a.out_wave_origin, (Index)a.n, i, wave_o);
+    store_out<int32_t, R>(a.out_occ_origin, i, occ_o);
+    store_out<int32_t, R>(a.out_wave_origin, i, wave_o);
   }
 }
 
