@@ -663,6 +663,9 @@ def main():
             args.records, 500, 2000)
         out["record_stream_GBps_at_%d_records" % args.large_records] = (
             device_info.record_stream_gbps(args.large_records, 20, 40))
+        # and for the launch with seven destinations (147 bytes per record)
+        out["record_stream_GBps_seven_destinations_at_%d_records" % args.records] = (
+            device_info.record_stream_multi_gbps(args.records, 7))
         # yardstick for the MLP: the vendor library's fp32 GEMM (+ bias) on one hidden
         # layer's shape, activations through HBM
         torch.backends.cuda.matmul.allow_tf32 = False

@@ -89,6 +89,8 @@ _SIGNATURES = {
     "hbt_measure_copy_gbps": (C.c_int, [C.c_size_t, C.POINTER(C.c_double)]),
     "hbt_measure_record_stream_gbps": (C.c_int, [C.c_int64, C.c_int, C.c_int,
                                                  C.POINTER(C.c_double)]),
+    "hbt_measure_record_stream_multi_gbps": (C.c_int, [C.c_int64, C.c_int32, C.c_int, C.c_int,
+                                                       C.POINTER(C.c_double)]),
 }
 
 # Entry points added after the first release of the ABI; bound when present.

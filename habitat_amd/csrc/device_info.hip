@@ -91,6 +91,38 @@ __global__ __launch_bounds__(128) void record_stream_kernel(const StreamArgs a) 
   __builtin_nontemporal_store((uint8_t)s, a.out_status + i);
 }
 
+struct MultiStreamArgs {
+  const int32_t* ints[5];
+  const double* dbls[4];
+  double* out_time;     // [n_dest][n]
+  int32_t* out_occ;     // [n_dest][n]
+  uint8_t* out_status;  // [n_dest][n]
+  int32_t* out_occ_origin;
+  uint32_t n;
+  int32_t n_dest;
+};
+
+// The data movement of a launch with several destinations: the record read
+// once, per destination one fp64, one int32 and one byte written to that
+// destination's rows, the origin occupancy once.
+__global__ __launch_bounds__(128) void record_stream_multi_kernel(const MultiStreamArgs a) {
+  const uint32_t i = blockIdx.x * 128u + threadIdx.x;
+  if (i >= a.n) return;
+  int32_t s = 0;
+  double d = 0;
+#pragma unroll
+  for (int k = 0; k < 5; ++k) s += __builtin_nontemporal_load(a.ints[k] + i);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) d += __builtin_nontemporal_load(a.dbls[k] + i);
+  for (int j = 0; j < a.n_dest; ++j) {
+    const size_t at = (size_t)j * a.n + i;
+    __builtin_nontemporal_store(d + j, a.out_time + at);
+    __builtin_nontemporal_store(s + j, a.out_occ + at);
+    __builtin_nontemporal_store((uint8_t)(s + j), a.out_status + at);
+  }
+  __builtin_nontemporal_store(s, a.out_occ_origin + i);
+}
+
 struct Timer {
   hipEvent_t e0 = nullptr, e1 = nullptr;
   bool ok = false;
@@ -294,6 +326,56 @@ int hbt_measure_record_stream_gbps(int64_t n, int warmup, int launches, double* 
     return rc;
   }
   *out_gbps = 68.0 * (double)n * launches / (ms * 1e6);  // the kernel's algorithmic bytes
+  return HBT_OK;
+}
+
+int hbt_measure_record_stream_multi_gbps(int64_t n, int32_t n_dest, int warmup, int launches,
+                                         double* out_gbps) {
+  using namespace hbt;
+  if (n < 2 || n > ((int64_t)1 << 28) || n_dest < 1 || n_dest > 64 || warmup < 0 ||
+      launches <= 0 || out_gbps == nullptr)
+    return HBT_EINVAL;
+  const size_t col4 = ((size_t)n * 4 + 255) & ~(size_t)255, col8 = ((size_t)n * 8 + 255) & ~(size_t)255;
+  const size_t rows8 = ((size_t)n * 8 * n_dest + 255) & ~(size_t)255;
+  const size_t rows4 = ((size_t)n * 4 * n_dest + 255) & ~(size_t)255;
+  const size_t total = 6 * col4 + 4 * col8 + rows8 + rows4 + (size_t)n * n_dest;
+  char* base = nullptr;
+  if (hipMalloc(reinterpret_cast<void**>(&base), total) != hipSuccess) {
+    (void)hipGetLastError();
+    return HBT_ENOMEM;
+  }
+  MultiStreamArgs a{};
+  char* p = base;
+  for (int k = 0; k < 5; ++k) { a.ints[k] = reinterpret_cast<const int32_t*>(p); p += col4; }
+  for (int k = 0; k < 4; ++k) { a.dbls[k] = reinterpret_cast<const double*>(p); p += col8; }
+  a.out_occ_origin = reinterpret_cast<int32_t*>(p); p += col4;
+  a.out_time = reinterpret_cast<double*>(p); p += rows8;
+  a.out_occ = reinterpret_cast<int32_t*>(p); p += rows4;
+  a.out_status = reinterpret_cast<uint8_t*>(p);
+  a.n = (uint32_t)n;
+  a.n_dest = n_dest;
+  const unsigned blocks = (unsigned)((n + 127) / 128);
+  Timer t;
+  int rc = t.ok ? HBT_OK : HBT_EHIP;
+  float ms = 0.f;
+  if (rc == HBT_OK && hipMemsetAsync(base, 0, total, nullptr) != hipSuccess) rc = HBT_EHIP;
+  if (rc == HBT_OK) {
+    for (int i = 0; i < warmup; ++i)
+      hipLaunchKernelGGL(record_stream_multi_kernel, dim3(blocks), dim3(128), 0, nullptr, a);
+    (void)hipEventRecord(t.e0, nullptr);
+    for (int i = 0; i < launches; ++i)
+      hipLaunchKernelGGL(record_stream_multi_kernel, dim3(blocks), dim3(128), 0, nullptr, a);
+    (void)hipEventRecord(t.e1, nullptr);
+    if (hipEventSynchronize(t.e1) != hipSuccess ||
+        hipEventElapsedTime(&ms, t.e0, t.e1) != hipSuccess || hipGetLastError() != hipSuccess)
+      rc = HBT_EHIP;
+  }
+  (void)hipFree(base);
+  if (rc != HBT_OK) {
+    (void)hipGetLastError();
+    return rc;
+  }
+  *out_gbps = (56.0 + 13.0 * n_dest) * (double)n * launches / (ms * 1e6);
   return HBT_OK;
 }
 

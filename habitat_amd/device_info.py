@@ -63,6 +63,16 @@ def record_stream_gbps(records, warmup=2000, launches=2000):
     return v.value
 
 
+def record_stream_multi_gbps(records, n_dest, warmup=500, launches=500):
+    """GB/s (52 + 4 + 13 x n_dest bytes per record) of a kernel doing only the
+    loads and stores of wave scaling to `n_dest` destinations in one launch."""
+    v = ctypes.c_double(0)
+    _lib.check(_lib.lib().hbt_measure_record_stream_multi_gbps(records, n_dest, warmup, launches,
+                                                               ctypes.byref(v)),
+               "hbt_measure_record_stream_multi_gbps")
+    return v.value
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--device", type=int, default=0)

@@ -369,12 +369,18 @@ int hbt_mlp_forward_static(hbt_mlp *mlp, const double *raw_features, int64_t n, 
  * no arithmetic, `launches` times after `warmup` untimed ones, and reports
  * 68 bytes per record over the launch time: the data-movement ceiling the
  * wave-scaling kernel can be held against at that size.
+ * hbt_measure_record_stream_multi_gbps does the same for a launch with n_dest
+ * destinations (the record read once, 13 bytes written per destination to
+ * that destination's rows, the origin occupancy once) and reports 52 + 4 + 13
+ * x n_dest bytes per record over the launch time.
  */
 int hbt_local_device_spec(int device, hbt_device_spec *out, char *name, size_t name_len);
 int hbt_measure_fp32_fma_gflops(int iters, double *out_gflops);
 int hbt_measure_fp32_mfma_gflops(int iters, double *out_gflops);
 int hbt_measure_copy_gbps(size_t bytes, double *out_gbps);
 int hbt_measure_record_stream_gbps(int64_t n, int warmup, int launches, double *out_gbps);
+int hbt_measure_record_stream_multi_gbps(int64_t n, int32_t n_dest, int warmup, int launches,
+                                         double *out_gbps);
 
 #ifdef __cplusplus
 }
