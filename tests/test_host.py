@@ -406,3 +406,30 @@ def test_record_cache_fingerprint_sees_in_place_changes():
     passes[1].kernels.pop(0)
     passes[0].kernels.append(moved)
     assert _fingerprint(passes) == base
+
+
+def test_the_c_abi_from_plain_c99(tmp_path, built_library):
+    """include/habitat_mi.h is C: a C99 program compiled with -pedantic -Werror
+    links against the library and gets the host-side answers without Python."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    lib_dir = os.path.dirname(built_library)
+    exe = str(tmp_path / "abi_c99")
+    cmd = [gcc, "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror",
+           "-I", os.path.join(ROOT, "include"), "-o", exe,
+           os.path.join(ROOT, "tests", "native", "abi_c99.c"),
+           "-L", lib_dir, "-lhabitat_mi", "-Wl,-rpath," + lib_dir]
+    built = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert built.returncode == 0, built.stdout
+    import torch
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    env = dict(os.environ)
+    env["LD_LIBRARY_PATH"] = os.pathsep.join(
+        [torch_lib, "/opt/rocm/lib", env.get("LD_LIBRARY_PATH", "")])
+    run = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                         env=env, timeout=120)
+    assert run.returncode == 0, (run.returncode, run.stdout)
+    assert run.stdout.startswith("ok:"), run.stdout
