@@ -244,12 +244,18 @@ class RuntimePredictor:
         remembered = self._predicted
         value = remembered.get(key)
         if value is not None:
-            remembered.move_to_end(key)
+            try:
+                remembered.move_to_end(key)
+            except KeyError:          # another thread has just dropped it
+                pass
             return value
         value = self._device_mlp().predict_one(features)
         remembered[key] = value
-        if len(remembered) > self.PREDICT_CACHE_ENTRIES:
-            remembered.popitem(last=False)
+        while len(remembered) > self.PREDICT_CACHE_ENTRIES:
+            try:
+                remembered.popitem(last=False)
+            except KeyError:          # another thread emptied it
+                break
         return value
 
     def predict_batch(self, raw_features, out=None, stream=None):
