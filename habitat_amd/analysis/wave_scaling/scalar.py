@@ -65,7 +65,9 @@ def scale_one(kernel, origin_device, dest_device, metadata_manager, metrics, loo
     pinned, device-visible record and a wait, about ten microseconds for a few
     hundred arithmetic operations, where the batched call spends a hundredth of
     a nanosecond per record.  Callers with many kernels should hand them over
-    together (Predictor.predict_operations)."""
+    together (Predictor.predict_operations), or keep this signature and use a
+    deferred strategy (wave_scaling/deferred.py), which launches once per set
+    of kernels."""
     nb, block, dyn, stat, regs, t_ns = kernel_fields(kernel)
     dest_regs = metadata_manager.kernel_registers_for(kernel, lookup_device or dest_device)
     record, time_ns, status, p_record, p_time, p_status = _call_state()
