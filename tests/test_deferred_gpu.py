@@ -85,6 +85,26 @@ def test_host_records_match_the_oracle_and_the_column_kernel(n):
     assert np.array_equal(out.status[0].cpu().numpy(), st)
 
 
+@pytest.mark.parametrize("pair", [("V100", "MI355X"), ("MI355X", "T4"), ("P100", "V100"),
+                                  ("V100", "MI355X_cdna")])
+def test_host_records_on_adversarial_field_values(pair):
+    """Zeros of both signs, subnormals, infinities, NaN, out-of-range integers:
+    the host-record kernel must write what the column kernel writes, bit for
+    bit, in every output (the column kernel is held against the oracle on the
+    same records elsewhere)."""
+    from test_wave_scale_gpu import adversarial_records
+    origin, dest = getattr(Device, pair[0]), getattr(Device, pair[1])
+    rec = adversarial_records(40_000, 123)
+    rc, t, st, oo, od = call_host_records(origin, dest, host_records(rec))
+    assert rc == 0
+    out = wave_scale(KernelRecords.from_numpy(rec), origin, [dest])
+    assert np.array_equal(out.time_ns[0].cpu().numpy(), t, equal_nan=True)
+    assert np.array_equal(out.status[0].cpu().numpy(), st)
+    assert np.array_equal(out.occ_origin.cpu().numpy(), oo)
+    assert np.array_equal(out.occ_dest[0].cpu().numpy(), od)
+    assert len(set(st.tolist())) >= 4          # the set does reach the statuses
+
+
 def test_host_records_arguments_and_streams():
     origin, dest = Device.V100, Device.T4
     lib = _lib.lib()
