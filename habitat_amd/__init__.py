@@ -51,6 +51,7 @@ _SUBMODULES = [
     "analysis.wave_scaling", "analysis.wave_scaling.common", "analysis.wave_scaling.metadata",
     "analysis.wave_scaling.resimplified", "analysis.wave_scaling.roofline",
     "analysis.wave_scaling.unified", "analysis.wave_scaling.batch", "analysis.wave_scaling.cdna",
+    "analysis.wave_scaling.deferred", "analysis.wave_scaling.scalar",
     "analysis.report", "analysis.sweep", "data", "device", "utils",
 ]
 

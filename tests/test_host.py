@@ -212,6 +212,7 @@ def test_habitat_alias_imports():
     from habitat.analysis.wave_scaling.resimplified import resimplified_wave_scaling  # noqa: F401
     from habitat.analysis.wave_scaling.roofline import roofline_wave_scaling  # noqa: F401
     from habitat.analysis.wave_scaling.unified import unified_wave_scaling  # noqa: F401
+    from habitat.analysis.wave_scaling.deferred import deferred_unified_wave_scaling  # noqa: F401
     from habitat.analysis.mlp.mlp import RuntimePredictor, LinearMLP, LSTMMLP, Conv2DMLP, BMMMLP  # noqa: F401
     from habitat.analysis.predictor import Predictor  # noqa: F401
     from habitat.analysis.kernels import MeasuredKernel, PredictedKernel, KernelInstance
