@@ -473,6 +473,13 @@ def test_local_device_description_and_measured_ceilings():
     assert m["fp32_fma_gflops"] <= props["peak_gflops_per_second"] <= 1.15 * m["fp32_fma_gflops"]
     assert props["peak_gflops_per_second"] == pytest.approx(157300 / 2, rel=0.02)
     assert m["fp32_mfma_gflops"] == pytest.approx(157300, rel=0.05)
+    # the data-movement yardsticks of wave scaling: one destination and seven
+    one = device_info.record_stream_gbps(1_000_000, 200, 200)
+    seven = device_info.record_stream_multi_gbps(1_000_000, 7, 100, 100)
+    assert 3000 < seven < one < 8000 * 1.03
+    from habitat_amd import _lib
+    v = __import__("ctypes").c_double(0)
+    assert _lib.lib().hbt_measure_record_stream_multi_gbps(1000, 0, 1, 1, v) == _lib.HBT_EINVAL
     # the reading as a compute-unit description: the GPU of the table's MI355X_cdna row
     from habitat_amd.analysis.wave_scaling.cdna import native_description
     native = native_description(dev).as_dict()
