@@ -74,6 +74,8 @@ _SIGNATURES = {
     "hbt_device_table_size": (C.c_int32, [_P]),
     "hbt_device_table_destroy": (None, [_P]),
     "hbt_wave_scale_sum": (C.c_int, [_P, C.c_int64] + [_P] * 12 + [C.c_int32, _P, _P, _P]),
+    "hbt_wave_scale_sum_ordered": (C.c_int, [_P, C.c_int64] + [_P] * 12 + [C.c_int32, _P, _P, _P,
+                                                                            _P]),
     "hbt_roofline_gamma": (C.c_int, [C.POINTER(DeviceSpec), C.POINTER(DeviceSpec), C.c_int64,
                                      _P, _P, _P, _P, _P, _P]),
     "hbt_ratio_scale": (C.c_int, [_P, C.c_int32, C.c_int32, _P, C.c_int32, _P, _P, _P, _P, _P]),

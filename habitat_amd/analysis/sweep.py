@@ -9,8 +9,9 @@ analysis/run_time.py:50-58, analysis/predictor.py:111-148)
 
 `overhead_p = max(0, ms_p * 1e6 - sum_k t_k)` depends on the origin only, so it
 is computed once on the host.  The per-destination parts run on the GPU: one
-hbt_wave_scale_sum launch over all kernel records of the trace (scaled times
-are summed per pass on the fly and never written out), one MLP launch per
+hbt_wave_scale_sum_ordered launch over all kernel records of the trace (scaled
+times are summed per pass on the fly, in the kernels' order, and never written
+out), one MLP launch per
 operation kind over (destinations + origin) x distinct feature rows (a network
 repeats layer shapes: ResNet-50's 53 convolutions have 23 distinct rows), and
 hbt_ratio_scale for the ratio, clamp and sum.
@@ -96,6 +97,11 @@ class TracePlan:
         self.n_seg = max(len(owners), 1)
         self.segment = (torch.tensor(segment, dtype=torch.int32, device=self.gpu)
                         if kernels else None)
+        # a pass's kernels are consecutive records: pass p is the run
+        # [segment_start[p], segment_start[p + 1]), summed in that order
+        counts = np.bincount(np.asarray(segment, np.int64), minlength=self.n_seg)
+        self.segment_start = torch.tensor(np.concatenate([[0], np.cumsum(counts)]),
+                                          dtype=torch.int64, device=self.gpu)
         self._records = {}
         self.special = {}
         for kind, idxs in special.items():
@@ -137,7 +143,10 @@ class TracePlan:
 class SweepCall:
     """A prepared sweep: `launch()` enqueues its kernels on the current stream
     and returns a TraceSweep of GPU tensors, without synchronising and without
-    reading anything back, so it can be repeated or captured in a HIP graph."""
+    reading anything back, so it can be repeated or captured in a HIP graph.
+    Launches of ONE prepared sweep must follow each other on one stream (or be
+    ordered otherwise): they share the workspace the scaled times pass through
+    and the side streams the networks run on."""
 
     def __init__(self, plan, dests, device_features):
         from habitat_amd.analysis import predictor as P
@@ -160,7 +169,10 @@ class SweepCall:
                 table = DeviceTable(P.occupancy_device(plan.origin, plan.mode),
                                     [P.occupancy_device(dests[i], plan.mode) for i in idxs])
                 at = None if whole else torch.tensor(idxs, device=plan.gpu)
-                self.groups.append((rec, table, at))
+                # where the scaled times pass through on their way to the ordered sums
+                work = torch.empty((len(idxs), max(rec.n, 1)), dtype=torch.float64,
+                                   device=plan.gpu)
+                self.groups.append((rec, table, at, work))
         self.streams = [torch.cuda.Stream(plan.gpu) for _ in plan.special]   # default priority
         # The MLP input rows of every kind, (destinations + origin) x distinct
         # operation rows: they depend on the plan and the destinations only, so
@@ -199,15 +211,17 @@ class SweepCall:
         total = torch.full((D,), plan.const_ms, dtype=torch.float64, device=plan.gpu)
         if self.groups:
             if len(self.groups) == 1 and self.groups[0][2] is None:
-                rec, table, _ = self.groups[0]
-                res.pass_kernel_ns, res.bad_records = wave_scale_sum(rec, table, plan.segment,
-                                                                     plan.n_seg)
+                rec, table, _, work = self.groups[0]
+                res.pass_kernel_ns, res.bad_records = wave_scale_sum(
+                    rec, table, n_segments=plan.n_seg, segment_start=plan.segment_start,
+                    workspace=work)
             else:
                 res.pass_kernel_ns = torch.zeros((D, plan.n_seg), dtype=torch.float64,
                                                  device=plan.gpu)
                 res.bad_records = torch.zeros((D,), dtype=torch.int32, device=plan.gpu)
-                for rec, table, at in self.groups:
-                    sums, bad = wave_scale_sum(rec, table, plan.segment, plan.n_seg)
+                for rec, table, at, work in self.groups:
+                    sums, bad = wave_scale_sum(rec, table, n_segments=plan.n_seg,
+                                               segment_start=plan.segment_start, workspace=work)
                     res.pass_kernel_ns[at] = sums
                     res.bad_records[at] = bad
             total += res.pass_kernel_ns.sum(dim=1) / 1e6

@@ -172,13 +172,51 @@ class DeviceTable:
             pass
 
 
-def wave_scale_sum(records, table, segment=None, n_segments=1, stream=None):
+def wave_scale_sum(records, table, segment=None, n_segments=1, stream=None, segment_start=None,
+                   workspace=None):
     """Per destination of `table` and per segment, the sum of the scaled times
     of `records` (see hbt_wave_scale_sum).  `segment`: int32 GPU tensor [n] or
-    None.  Returns (sums [n_dest, n_segments] float64, bad [n_dest] int32), both
-    GPU tensors, not synchronised."""
+    None.  Or `segment_start`: int64 GPU tensor [n_segments + 1] when segment s
+    is the run of records [segment_start[s], segment_start[s + 1]): the times
+    are then added in the records' order, as the reference adds a pass's
+    kernels, without floating-point atomics (hbt_wave_scale_sum_ordered; the
+    scaled times pass through `workspace`, a float64 GPU tensor of n_dest x n
+    elements, allocated here when not given).
+    Returns (sums [n_dest, n_segments] float64, bad [n_dest] int32), both GPU
+    tensors, not synchronised."""
     if records.device != table.torch_device:
         raise ValueError("records and device table live on different GPUs")
+    if segment_start is not None:
+        if segment is not None:
+            raise ValueError("give segment or segment_start, not both")
+        if (segment_start.dtype != torch.int64 or segment_start.shape != (n_segments + 1,)
+                or segment_start.device != records.device):
+            raise TypeError("segment_start must be an int64 GPU tensor of length %d"
+                            % (n_segments + 1))
+        n_dest = len(table)
+        sums = torch.empty((n_dest, n_segments), dtype=torch.float64, device=records.device)
+        bad = torch.empty((n_dest,), dtype=torch.int32, device=records.device)
+        if workspace is None:
+            workspace = torch.empty((n_dest, max(records.n, 1)), dtype=torch.float64,
+                                    device=records.device)
+        elif (workspace.dtype != torch.float64 or workspace.numel() < n_dest * records.n
+              or workspace.device != records.device or not workspace.is_contiguous()):
+            raise TypeError("workspace must be a contiguous float64 GPU tensor of at least "
+                            "%d elements" % (n_dest * records.n))
+        if stream is None:
+            stream = torch.cuda.current_stream(records.device)
+        c = records.columns
+        with torch.cuda.device(records.device):
+            rc = _lib.lib().hbt_wave_scale_sum_ordered(
+                table.handle, records.n,
+                _ptr(c["num_blocks"]), _ptr(c["block_size"]), _ptr(c["dynamic_smem"]),
+                _ptr(c["static_smem"]), _ptr(c["regs_per_thread"]), _ptr(records.dest_regs),
+                _ptr(c["run_time_ns"]), _ptr(c["flop_sp_efficiency"]),
+                _ptr(c["dram_read_bytes"]), _ptr(c["dram_write_bytes"]),
+                _ptr(records.has_metrics), _ptr(segment_start.contiguous()), n_segments,
+                _ptr(workspace), _ptr(sums), _ptr(bad), ctypes.c_void_p(stream.cuda_stream))
+        _lib.check(rc, "hbt_wave_scale_sum_ordered")
+        return sums, bad
     if segment is not None and (segment.dtype != torch.int32 or segment.shape != (records.n,)
                                 or segment.device != records.device):
         raise TypeError("segment must be an int32 GPU tensor of length %d" % records.n)

@@ -72,6 +72,7 @@ struct SumArgs {
   const int32_t* segment;      // nullable: all records in segment 0
   double* out_sum;             // [n_dest][n_segments]
   int32_t* out_bad;            // [n_dest], nullable
+  double* work;                // ORDERED: [n_dest][n]
   const DestArgs* dests;
   OriginArgs origin;
 };
@@ -86,7 +87,10 @@ __global__ void fill_zero_kernel(double* sums, int64_t n_sums, int32_t* bad, int
 // wavefront, consecutive records of the same segment are summed with a
 // segmented scan and the last lane of each run adds the run's total to the
 // segment's sum, per destination.
-template <int MODEL>
+// ORDERED: no sums here; each scaled time (+0 where the reference would raise)
+// goes to a.work[destination][record] for segment_sum_ordered_kernel to add up
+// in the records' order.
+template <int MODEL, bool ORDERED>
 __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a) {
   const int d0 = blockIdx.y * kSumGroup;
   const int d1 = d0 + kSumGroup < a.n_dest ? d0 + kSumGroup : a.n_dest;
@@ -107,7 +111,7 @@ __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a)
   r.rd = a.dram_read_bytes[j];
   r.wr = a.dram_write_bytes[j];
   // lanes past the end form a run of their own so that they never swallow a tail
-  const int32_t seg = in_range ? (a.segment != nullptr ? a.segment[j] : 0) : -1;
+  const int32_t seg = (in_range && !ORDERED) ? (a.segment != nullptr ? a.segment[j] : 0) : -1;
 
   RecordMid m = origin_part<MODEL>(a.origin, r);
   if (__builtin_expect(m.redo_gflops, 0))
@@ -140,6 +144,10 @@ __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a)
       const unsigned long long bad = __ballot(in_range && o.status != HBT_ST_OK);
       if (lane == 0 && bad != 0) atomicAdd(a.out_bad + d, (int32_t)__popcll(bad));
     }
+    if (ORDERED) {
+      if (in_range) a.work[(int64_t)d * a.n + i] = v;
+      continue;
+    }
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
       const double other = __shfl_up(v, off);
@@ -148,6 +156,34 @@ __global__ __launch_bounds__(kBlock) void wave_scale_sum_kernel(const SumArgs a)
     }
     if (adds) unsafeAtomicAdd(a.out_sum + (int64_t)d * a.n_segments + seg, v);
   }
+}
+
+struct OrderedSumArgs {
+  int64_t n;
+  int32_t n_segments;
+  const double* work;            // [n_dest][n], from wave_scale_sum_kernel<., true>
+  const int64_t* segment_start;  // [n_segments + 1]
+  double* out_sum;               // [n_dest][n_segments]
+};
+
+// One thread per (segment, destination = blockIdx.y): it adds the segment's
+// scaled times one after the other in the records' order, as the reference
+// adds a pass's kernels (run_time.py:50-58).  No floating-point atomics: the
+// sum is the same every time, and the same as a sequential sum of the
+// per-record kernel's times.  (The loads do not depend on the running sum, so
+// they run ahead of the additions.)
+__global__ __launch_bounds__(kBlock) void segment_sum_ordered_kernel(const OrderedSumArgs a) {
+  const int s = blockIdx.x * kBlock + threadIdx.x;
+  if (s >= a.n_segments) return;
+  // (clamped to the columns: a wrong boundary must not become a stray read)
+  int64_t begin = a.segment_start[s], end = a.segment_start[s + 1];
+  begin = begin < 0 ? 0 : begin;
+  end = end > a.n ? a.n : end;
+  const double* v = a.work + (int64_t)blockIdx.y * a.n;
+  double sum = 0.0;
+#pragma unroll 8
+  for (int64_t j = begin; j < end; ++j) sum += v[j];
+  a.out_sum[(int64_t)blockIdx.y * a.n_segments + s] = sum;
 }
 
 struct GammaArgs {
@@ -355,8 +391,74 @@ int hbt_wave_scale_sum(const hbt_device_table* table, int64_t n, const int32_t* 
   a.origin = table->origin;
   const dim3 grid((unsigned)blocks, (unsigned)((table->n_dest + kSumGroup - 1) / kSumGroup));
   dev::with_model(table->model, [&](auto m) {
-    hipLaunchKernelGGL(wave_scale_sum_kernel<decltype(m)::value>, grid, dim3(kBlock), 0, stream, a);
+    hipLaunchKernelGGL((wave_scale_sum_kernel<decltype(m)::value, false>), grid, dim3(kBlock), 0,
+                       stream, a);
   });
+  return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
+}
+
+int hbt_wave_scale_sum_ordered(const hbt_device_table* table, int64_t n, const int32_t* num_blocks,
+                               const int32_t* block_size, const int32_t* dynamic_smem,
+                               const int32_t* static_smem, const int32_t* regs,
+                               const int32_t* dest_regs, const double* run_time_ns,
+                               const double* flop_sp_efficiency, const double* dram_read_bytes,
+                               const double* dram_write_bytes, const uint8_t* has_metrics,
+                               const int64_t* segment_start, int32_t n_segments, double* workspace,
+                               double* out_sum, int32_t* out_bad, void* hip_stream) {
+  using namespace hbt;
+  if (table == nullptr || n < 0 || n_segments <= 0 || out_sum == nullptr ||
+      segment_start == nullptr)
+    return HBT_EINVAL;
+  if (n > 0 && (!num_blocks || !block_size || !dynamic_smem || !static_smem || !regs ||
+                !run_time_ns || !flop_sp_efficiency || !dram_read_bytes || !dram_write_bytes ||
+                !workspace))
+    return HBT_EINVAL;
+  const int64_t blocks = (n + kBlock - 1) / kBlock;
+  if (blocks > 0x7fffffff || (int64_t)n_segments * table->n_dest > ((int64_t)1 << 38))
+    return HBT_ESIZE;
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    return HBT_EHIP;
+  }
+  if (device != table->device) return HBT_EINVAL;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  if (out_bad != nullptr) {
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((table->n_dest + kBlock - 1) / kBlock)),
+                       dim3(kBlock), 0, stream, static_cast<double*>(nullptr), (int64_t)0, out_bad,
+                       table->n_dest);
+    if (hipGetLastError() != hipSuccess) return HBT_EHIP;
+  }
+  if (n > 0) {
+    SumArgs a{};
+    a.n = n;
+    a.n_segments = n_segments;
+    a.n_dest = table->n_dest;
+    a.num_blocks = num_blocks; a.block_size = block_size; a.dynamic_smem = dynamic_smem;
+    a.static_smem = static_smem; a.regs = regs; a.dest_regs = dest_regs;
+    a.run_time_ns = run_time_ns; a.flop_sp_efficiency = flop_sp_efficiency;
+    a.dram_read_bytes = dram_read_bytes; a.dram_write_bytes = dram_write_bytes;
+    a.has_metrics = has_metrics;
+    a.out_bad = out_bad;
+    a.work = workspace;
+    a.dests = table->dests;
+    a.origin = table->origin;
+    const dim3 grid((unsigned)blocks, (unsigned)((table->n_dest + kSumGroup - 1) / kSumGroup));
+    dev::with_model(table->model, [&](auto m) {
+      hipLaunchKernelGGL((wave_scale_sum_kernel<decltype(m)::value, true>), grid, dim3(kBlock), 0,
+                         stream, a);
+    });
+    if (hipGetLastError() != hipSuccess) return HBT_EHIP;
+  }
+  OrderedSumArgs b{};
+  b.n = n;
+  b.n_segments = n_segments;
+  b.work = workspace;
+  b.segment_start = segment_start;
+  b.out_sum = out_sum;
+  hipLaunchKernelGGL(segment_sum_ordered_kernel,
+                     dim3((unsigned)((n_segments + kBlock - 1) / kBlock), (unsigned)table->n_dest),
+                     dim3(kBlock), 0, stream, b);
   return hipGetLastError() == hipSuccess ? HBT_OK : HBT_EHIP;
 }
 

@@ -242,6 +242,28 @@ int hbt_wave_scale_sum(const hbt_device_table *table, int64_t n, const int32_t *
                        double *out_sum, int32_t *out_bad, void *hip_stream);
 
 /*
+ * The same sums for segments that are runs of consecutive records, added up in
+ * the records' order like the reference's sequential sum over a pass's kernels
+ * (analysis/run_time.py:50-58): segment s holds the records
+ * [segment_start[s], segment_start[s + 1]) (device, [n_segments + 1], int64,
+ * non-decreasing, segment_start[n_segments] <= n; the caller guarantees that).
+ * No floating-point atomics: the scaled times go through `workspace` (device,
+ * [n_dest][n] doubles, the caller's; contents afterwards unspecified) and one
+ * thread per (segment, destination) adds them up in order, so out_sum[d][s] is
+ * the sequential fp64 sum of the times hbt_wave_scale writes for those records
+ * on d (a one-destination launch), bit for bit and the same on every run.
+ * Everything else as for hbt_wave_scale_sum.
+ */
+int hbt_wave_scale_sum_ordered(const hbt_device_table *table, int64_t n, const int32_t *num_blocks,
+                               const int32_t *block_size, const int32_t *dynamic_smem,
+                               const int32_t *static_smem, const int32_t *regs,
+                               const int32_t *dest_regs, const double *run_time_ns,
+                               const double *flop_sp_efficiency, const double *dram_read_bytes,
+                               const double *dram_write_bytes, const uint8_t *has_metrics,
+                               const int64_t *segment_start, int32_t n_segments, double *workspace,
+                               double *out_sum, int32_t *out_bad, void *hip_stream);
+
+/*
  * The roofline exponent alone, _roofline_gamma
  * (analysis/wave_scaling/roofline.py:68-104) with _ridge_point (:107-108), for n
  * records that all have their three metrics: out_gamma[n] fp64, NaN where the

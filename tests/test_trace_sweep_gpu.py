@@ -57,6 +57,49 @@ def test_fused_sums_match_oracle(n, n_seg, sorted_segments):
           "error vs oracle %.3g (bound 1e-06)" % (n, n_seg, len(dests), worst))
 
 
+@pytest.mark.parametrize("n,n_seg", [(1, 1), (900, 245), (5000, 3), (4097, 300), (70_000, 64)])
+def test_ordered_sums_are_the_sequential_sums_bit_for_bit(n, n_seg):
+    """hbt_wave_scale_sum_ordered adds a segment's scaled times in the records'
+    order, as the reference adds a pass's kernels (run_time.py:50-58): the
+    result must equal the sequential fp64 sum of the per-record kernel's times,
+    bit for bit, whatever the segment lengths (empty ones included), and come
+    out the same on every call; the atomic version agrees with it to rounding."""
+    origin = Device.V100
+    rec, _ = synthetic.kernel_records(n, origin, seed=n + n_seg, metrics_fraction=0.5)
+    rng = np.random.default_rng(n)
+    cuts = np.sort(rng.integers(0, n + 1, n_seg - 1))
+    start = np.concatenate([[0], cuts, [n]]).astype(np.int64)      # some segments are empty
+    segment = np.repeat(np.arange(n_seg, dtype=np.int32), np.diff(start))
+    dests = [Device.MI355X, Device.T4, Device.P100, Device.P4000, Device.V100]
+    kr = KernelRecords.from_numpy(rec)
+    table = DeviceTable(origin, dests)
+    start_gpu = torch.from_numpy(start).cuda()
+    sums, bad = wave_scale_sum(kr, table, n_segments=n_seg, segment_start=start_gpu)
+    again, bad_again = wave_scale_sum(kr, table, n_segments=n_seg, segment_start=start_gpu)
+    assert torch.equal(sums, again) and torch.equal(bad, bad_again)
+    # (one destination per launch: a launch with several forms gamma above the
+    # ridge as a product and can differ from these in the last bits)
+    single = [wave_scale(kr, origin, [d]) for d in dests]
+    t = np.stack([o.time_ns[0].cpu().numpy() for o in single])
+    st = np.stack([o.status[0].cpu().numpy() for o in single])
+    got = sums.cpu().numpy()
+    for di in range(len(dests)):
+        for s in range(n_seg):
+            want = 0.0
+            for j in range(start[s], start[s + 1]):
+                if st[di, j] == 0:
+                    want += t[di, j]
+            assert got[di, s] == want, (di, s)
+        assert int(bad[di]) == int((st[di] != 0).sum())
+    atomic, atomic_bad = wave_scale_sum(kr, table, torch.from_numpy(segment).cuda(), n_seg)
+    assert torch.equal(atomic_bad, bad)
+    np.testing.assert_allclose(atomic.cpu().numpy(), got, rtol=1e-12, atol=0)
+    # boundaries outside the columns are clamped, not followed
+    wild = torch.tensor([-5] + [n + 1000] * n_seg, dtype=torch.int64, device="cuda")
+    clamped, _ = wave_scale_sum(kr, table, n_segments=n_seg, segment_start=wild)
+    assert bool(torch.all(torch.isfinite(clamped)))
+
+
 def test_fused_sums_count_records_the_reference_would_raise_on(kat):
     base = dict(kat["scaling_record"])
     rows = [dict(base, num_blocks=10, dynamic_smem=60000),        # status 2 on V100
