@@ -591,6 +591,59 @@ def main():
 
     attempt("scalar_strategy", scalar_section)
 
+    # ---------------- records and results in HOST memory (PCIe inclusive) ----------------
+    def host_records_section():
+        import ctypes
+        from habitat_amd.analysis.wave_scaling.deferred import RECORD_DTYPE
+        host = np.zeros(args.records, RECORD_DTYPE)
+        for src, dst in (("num_blocks", "num_blocks"), ("block_size", "block_size"),
+                         ("dynamic_smem", "dynamic_smem"), ("static_smem", "static_smem"),
+                         ("regs_per_thread", "regs"), ("run_time_ns", "run_time_ns"),
+                         ("flop_sp_efficiency", "flop_sp_efficiency"),
+                         ("dram_read_bytes", "dram_read_bytes"),
+                         ("dram_write_bytes", "dram_write_bytes")):
+            host[dst] = rec[src]
+        host["dest_regs"], host["has_metrics"] = -1, 1
+        t_ns, st = np.empty(args.records), np.empty(args.records, np.uint8)
+        occ_o, occ_d = np.empty(args.records, np.int32), np.empty(args.records, np.int32)
+        fn = _lib.lib().hbt_wave_scale_host_records
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+        def call(n):
+            rc = fn(ctypes.byref(origin.spec), ctypes.byref(dest.spec), n,
+                    ctypes.c_void_p(host.ctypes.data), ctypes.c_void_p(t_ns.ctypes.data),
+                    ctypes.c_void_p(st.ctypes.data), ctypes.c_void_p(occ_o.ctypes.data),
+                    ctypes.c_void_p(occ_d.ctypes.data), stream)
+            if rc != 0:
+                raise RuntimeError("hbt_wave_scale_host_records: %d" % rc)
+
+        def rate(n, reps):
+            call(n)
+            best = float("inf")
+            for _ in range(reps):
+                t0 = time.perf_counter()
+                call(n)
+                best = min(best, time.perf_counter() - t0)
+            return best
+        small = rate(900, 200)
+        whole = rate(args.records, 5)
+        # the same records through the column kernel: results must be identical
+        torch.cuda.synchronize()
+        same = (np.array_equal(t_ns, out.time_ns[0].cpu().numpy(), equal_nan=True) and
+                np.array_equal(occ_d, out.occ_dest[0].cpu().numpy()) and
+                np.array_equal(occ_o, out.occ_origin.cpu().numpy()))
+        return {"call_us_900_records": small * 1e6,
+                "records_per_s_900": 900 / small,
+                "records_per_s_%d" % args.records: args.records / whole,
+                "GBps_host_in_plus_out": (64 + 17) * args.records / whole / 1e9,
+                "equal_to_the_column_kernel": bool(same),
+                "what": "hbt_wave_scale_host_records: 64-byte records in host memory in, "
+                        "time + status + two occupancies in host memory out (17 bytes), "
+                        "through the library's pinned staging block, host copies and the "
+                        "wait included; best of 200 / 5 calls"}
+
+    attempt("host_records", host_records_section)
+
     # ---------------- the same kernel beyond the last-level cache ----------------
     def large_section(n_records=None):
         big = KernelRecords.from_numpy(tile_records(rec, n_records or args.large_records))

@@ -10,7 +10,14 @@
 //                        (analyzer/habitat/analysis/predictor.py:116-124).
 //                        Scaled times never reach HBM: traffic is the record
 //                        columns once per destination row of the grid (they stay
-//                        in L2) plus 8 bytes per (destination, segment).
+//                        in L2) plus 8 bytes per (destination, segment).  Sums of
+//                        runs that span wavefronts meet in floating-point atomics.
+//   hbt_wave_scale_sum_ordered
+//                        the same sums for segments that are runs of consecutive
+//                        records, added in the records' order as the reference
+//                        adds them, without atomics: the scaled times pass
+//                        through a caller's workspace and one thread per
+//                        (segment, destination) adds them up.
 //   hbt_ratio_scale      per destination and MLP-predicted operation:
 //                        run_time_ms * pred_dest / pred_origin, negative -> 0
 //                        (predictor.py:132-148 and :182,218,238,283), the
