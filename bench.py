@@ -23,6 +23,8 @@ inputs resident in HBM.  Prints ONE JSON line:
   mlp           the fused MFMA MLP (configs[2], conv2d, 1 M rows): rows/s, its
                 roofline against fp32 MFMA peak and a torch-CPU fp32 baseline
   scalar_strategy  the reference's one-kernel strategy call through the same kernel
+  host_records  the same records as an array of structures in HOST memory, results
+                back in host memory, copies and wait included
   sweep         configs[4]: one ResNet-50-shaped trace predicted for 256 devices
                 (fused per-pass sums + MLP rows + ratio kernel), eager and as a
                 replayed HIP graph, next to the per-device CPU path

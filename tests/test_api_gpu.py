@@ -465,14 +465,15 @@ def test_local_device_description_and_measured_ceilings():
     # mem_bandwidth_gb, base_clock_mhz, peak_gflops_per_second), held against
     # what the box measures and what is published for the MI355X: the bandwidth
     # lies between the measured copy rate and the published 8 TB/s (8192 GB/s
-    # by the clocks), the clock in 2.0-2.5 GHz, the vector fp32 peak within 15 %
-    # above the measured FMA rate and at half the published 157.3 TFLOP/s,
-    # which counts packed fp32 or the matrix cores.
+    # by the clocks), the clock in 2.0-2.5 GHz, the vector fp32 peak at most 30 %
+    # above the measured FMA rate (10 % on the boxes seen so far; the margin is
+    # for one that runs below its clock) and at half the published 157.3
+    # TFLOP/s, which counts packed fp32 or the matrix cores.
     assert m["copy_gbps"] < props["mem_bandwidth_gb"] <= 8000 * 1.03
     assert 2000 <= props["base_clock_mhz"] <= 2500
-    assert m["fp32_fma_gflops"] <= props["peak_gflops_per_second"] <= 1.15 * m["fp32_fma_gflops"]
+    assert m["fp32_fma_gflops"] <= props["peak_gflops_per_second"] <= 1.30 * m["fp32_fma_gflops"]
     assert props["peak_gflops_per_second"] == pytest.approx(157300 / 2, rel=0.02)
-    assert m["fp32_mfma_gflops"] == pytest.approx(157300, rel=0.05)
+    assert m["fp32_mfma_gflops"] == pytest.approx(157300, rel=0.15)    # measured: 155 000
     # the data-movement yardsticks of wave scaling: one destination and seven
     one = device_info.record_stream_gbps(1_000_000, 200, 200)
     seven = device_info.record_stream_multi_gbps(1_000_000, 7, 100, 100)
