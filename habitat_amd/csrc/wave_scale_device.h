@@ -101,7 +101,9 @@ __device__ __forceinline__ double exp2_poly(double x) {
 // division it replaces: q = x * (1/c) is within an ulp of the quotient, the
 // remainder x - q*c is exact in an FMA, and adding remainder * (1/c) back
 // rounds to the nearest double (Markstein's correction; checked against `/`
-// on 4e8 operands for each constant used here).  Valid where div_const_safe
+// on 1e9 operands for each constant used here).  One difference: x = -0.0
+// comes back as +0.0 (the zero remainder is positive); the FLOP count this
+// feeds is only compared with 1e-9, which no zero passes.  Valid where div_const_safe
 // holds; elsewhere the remainder could underflow or overflow and the caller
 // must divide for real.
 template <class C>
