@@ -12,6 +12,11 @@
 //   arith_div_const   div_const<C>(x) == x / C bit for bit wherever
 //                     div_const_safe(x), for C = 100 and 1e9 (but for the sign
 //                     of a zero, counted apart)
+//   arith_occupancy_lattice  the 32-bit occupancy models the kernels run
+//                     (occupancy_fast and its lean forms, occupancy_cdna in 32 bits)
+//                     against the 64-bit models with plain division
+//                     (occupancy_core, occupancy_cdna<true>) on a lattice of
+//                     launch configurations of one device
 //   arith_exp2        largest relative error of exp2_poly against exp2 on a grid
 //   arith_exp2_at     exp2_poly at given points (saturation, NaN)
 #include <hip/hip_runtime.h>
@@ -128,6 +133,54 @@ __global__ __launch_bounds__(kThreads) void div_const_kernel(u64 n, u64 seed, Re
   if (zero_sign != 0) atomicAdd(&rep->first_b, zero_sign);
 }
 
+// The lattice: block sizes -1..1100, registers per thread 0..300 and 65535
+// (what a uint16_t can hold at most), shared memory -600..600 bytes one by one
+// and from there to 70 000 every size that is 0, 1, 2, 127, 128, 254 or 255
+// above a multiple of 256 (all allocation granules are multiples of 256).
+constexpr int kLatticeBlocks = 1102, kLatticeRegs = 302;
+constexpr int kLatticeSmemDense = 1201, kLatticeSmemRows = 271;
+constexpr int kLatticeSmem = kLatticeSmemDense + 7 * kLatticeSmemRows;
+
+__device__ int32_t lattice_smem(int idx) {
+  if (idx < kLatticeSmemDense) return idx - 600;
+  const int j = idx - kLatticeSmemDense;
+  const int residue[7] = {0, 1, 2, 127, 128, 254, 255};
+  return 768 + (j / 7) * 256 + residue[j % 7];
+}
+
+// blockIdx.x: block size, blockIdx.y: registers; the threads stride over the
+// shared-memory sizes.  `variants`: bit 0 occupancy_fast, 1 its lean form, 2 the
+// lean form with the cc 6.0 re-check by select, 3 occupancy_cdna in 32 bits,
+// 4 its lean form.
+__global__ __launch_bounds__(kThreads) void occupancy_lattice_kernel(const OccDevice d,
+                                                                     uint32_t variants,
+                                                                     Report* rep) {
+  const int32_t block = (int32_t)blockIdx.x - 1;
+  const int32_t regs = blockIdx.y == kLatticeRegs - 1 ? 65535 : (int32_t)blockIdx.y;
+  u64 checked = 0, bad = 0, bad_a = 0, bad_b = 0;
+  for (int idx = threadIdx.x; idx < kLatticeSmem; idx += kThreads) {
+    const int32_t smem = lattice_smem(idx);
+    const SmemAlloc sm = smem_alloc(smem);
+    const int32_t want = (d.flags & kCdna) ? occupancy_cdna<true>(d, block, smem, regs)
+                                           : occupancy_core(d, block, smem, regs);
+    uint32_t wrong = 0;
+    if ((variants & 1) && occupancy_fast<false, false>(d, block, sm, regs) != want) wrong |= 1;
+    if ((variants & 2) && occupancy_fast<true, false>(d, block, sm, regs) != want) wrong |= 2;
+    if ((variants & 4) && occupancy_fast<true, true>(d, block, sm, regs) != want) wrong |= 4;
+    if ((variants & 8) && occupancy_cdna<false, false>(d, block, smem, regs) != want) wrong |= 8;
+    if ((variants & 16) && occupancy_cdna<false, true>(d, block, smem, regs) != want) wrong |= 16;
+    if (wrong != 0) {
+      if (bad == 0) {
+        bad_a = ((u64)(uint32_t)block << 32) | (uint32_t)smem;
+        bad_b = ((u64)(uint32_t)regs << 32) | wrong;
+      }
+      ++bad;
+    }
+    ++checked;
+  }
+  note(rep, checked, bad, bad_a, bad_b);
+}
+
 struct Exp2Report {
   u64 worst_err_bits;  // the largest relative error, as the bits of a double
   u64 checked;
@@ -230,6 +283,31 @@ int arith_div_const(int64_t which, u64 n, u64 seed, u64* out4) {
     hipLaunchKernelGGL(div_const_kernel<C1e9>, grid, dim3(kThreads), 0, 0, n, seed, rep.p);
   else
     return -1;
+  if (hipGetLastError() != hipSuccess) return -2;
+  return fetch(rep.p, out4);
+}
+
+// The occupancy models of one device on the lattice.  out4 = {configurations
+// checked, mismatches, (block << 32 | shared memory) and (registers << 32 |
+// variants that differ) of one mismatch}; *variants_run = the variants that
+// apply to this device (bits as in occupancy_lattice_kernel).
+int arith_occupancy_lattice(const hbt_device_spec* spec, uint32_t* variants_run, u64* out4) {
+  if (spec == nullptr) return -1;  // (a spec hbt_device_spec_check accepts: the caller's part)
+  const OccDevice d = make_occ_device(*spec);
+  uint32_t variants = 0;
+  if (d.flags & kCdna) {
+    if (d.fast_ok()) variants |= 8;
+    if (d.cdna_lean_ok()) variants |= 16;
+  } else {
+    if (d.fast_ok()) variants |= 1;
+    if (d.lean_ok()) variants |= 2;
+    if (d.lean_gp_ok()) variants |= 4;
+  }
+  *variants_run = variants;
+  DeviceBuffer<Report> rep(1);
+  if (rep.p == nullptr || hipMemset(rep.p, 0, sizeof(Report)) != hipSuccess) return -1;
+  hipLaunchKernelGGL(occupancy_lattice_kernel, dim3(kLatticeBlocks, kLatticeRegs), dim3(kThreads),
+                     0, 0, d, variants, rep.p);
   if (hipGetLastError() != hipSuccess) return -2;
   return fetch(rep.p, out4);
 }

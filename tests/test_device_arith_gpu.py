@@ -32,6 +32,7 @@ def arith():
     lib.arith_exp2.argtypes = [ctypes.c_double, ctypes.c_double, ctypes.c_uint64,
                                ctypes.POINTER(ctypes.c_double)]
     lib.arith_exp2_at.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
+    lib.arith_occupancy_lattice.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint32), u64p]
     return lib
 
 
@@ -101,3 +102,42 @@ def test_power_of_two_polynomial(arith):
     assert np.all(y[9:12] == 0.0)
     assert np.isnan(y[12])
     assert abs(y[13] / 2 ** 0.5 - 1) < 1e-13 and abs(y[14] / 2 ** -0.5 - 1) < 1e-13
+
+
+def test_32bit_occupancy_models_equal_the_64bit_ones_on_a_lattice(arith, occupancy_golden):
+    """Every variant of the occupancy model the kernels can run for a device
+    (32-bit arithmetic with reciprocal divisions, with and without the
+    branches that are uniform over a launch) against the 64-bit model with
+    plain divisions, which the CPU tests hold against the compiled reference:
+    1102 block sizes x 302 register counts x 3098 shared-memory sizes per
+    device, for the 15 device descriptions of the reference-built fixture and
+    the compute-unit reading of the one that has one."""
+    from habitat_amd import DeviceProperties
+    from habitat_amd.analysis.wave_scaling.cdna import native_description
+    _, described = occupancy_golden
+    specs = []
+    for name, kwargs in described.items():
+        dev = DeviceProperties(name=name, **{k: v for k, v in kwargs.items() if k != "name"})
+        specs.append((name, dev))
+        native = native_description(dev)
+        if native.compute_capability != dev.compute_capability:
+            specs.append((name + " as compute units", native))
+            odd = dict(native.as_dict(), warp_size=48)     # not a power of two: no lean form
+            specs.append((name + " as compute units, 48 lanes",
+                          DeviceProperties(name=name + "_48", **odd)))
+    total, seen = 0, 0
+    for name, dev in specs:
+        out = (ctypes.c_uint64 * 4)()
+        variants = ctypes.c_uint32(0)
+        assert arith.arith_occupancy_lattice(ctypes.addressof(dev.spec), ctypes.byref(variants),
+                                             out) == 0, name
+        checked, bad = out[0], out[1]
+        assert checked == 1102 * 302 * 3098
+        assert bad == 0, "%s: block %d smem %d regs %d variants %#x" % (
+            name, np.int32(out[2] >> 32), np.int32(out[2] & 0xffffffff), out[3] >> 32,
+            out[3] & 0xff)
+        total += checked * bin(variants.value).count("1")
+        seen |= variants.value
+    print("occupancy lattice: %d descriptions, %.3g (configuration, variant) pairs, variants %#x" %
+          (len(specs), total, seen), flush=True)
+    assert seen == 0x1f       # every variant ran for some device
