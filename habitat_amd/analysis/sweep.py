@@ -229,9 +229,9 @@ class SweepCall:
         else:
             res.pass_kernel_ns = torch.zeros((D, plan.n_seg), dtype=torch.float64, device=plan.gpu)
             res.bad_records = torch.zeros((D,), dtype=torch.int32, device=plan.gpu)
+        res.clamped_ops = torch.zeros((D,), dtype=torch.int32, device=plan.gpu)
         for side in self.streams:
             main.wait_stream(side)
-        res.clamped_ops = torch.zeros((D,), dtype=torch.int32, device=plan.gpu)
         for kind, (idxs, pred, op_feats, ms, op_row) in plan.special.items():
             res.special_ms[kind] = ratio_scale(preds[kind], ms, D, totals=total, op_row=op_row,
                                                clamped=res.clamped_ops)
