@@ -434,3 +434,17 @@ def test_the_c_abi_from_plain_c99(tmp_path, built_library):
                          env=env, timeout=120)
     assert run.returncode == 0, (run.returncode, run.stdout)
     assert run.stdout.startswith("ok:"), run.stdout
+
+
+def test_gpu_selftest_library_builds_and_exports_its_checkers():
+    """tests/native/device_arith.hip (the brute-force checkers of
+    tests/test_device_arith_gpu.py) cross-compiles for gfx950 and exports every
+    entry the GPU test binds; nothing is launched here."""
+    import ctypes
+    import subprocess
+    native = os.path.join(ROOT, "tests", "native")
+    subprocess.check_call(["make", "-s", "-C", native])
+    lib = ctypes.CDLL(os.path.join(native, "_build", "libdevice_arith.so"))
+    for name in ("arith_fast_div", "arith_ceil_div", "arith_div_const", "arith_exp2",
+                 "arith_exp2_at", "arith_occupancy_lattice"):
+        assert hasattr(lib, name), name
