@@ -13,7 +13,8 @@
 // library keeps per GPU (allocated on the first call there, kept until the
 // process ends); the kernel reads the records and writes the results straight
 // through it, so a call is one memcpy into the block, one launch, one wait and
-// one memcpy out.  The arithmetic is the code of wave_scale_device.h that the
+// one memcpy out; arrays longer than the block go through its two halves in
+// turn, the copies of one chunk beside the launch of the next.  The arithmetic is the code of wave_scale_device.h that the
 // column kernel runs.
 #include <hip/hip_runtime.h>
 
@@ -100,18 +101,22 @@ __global__ __launch_bounds__(kBlock) void wave_scale_records_kernel(const HostRe
   }
 }
 
-// The staging block of one GPU: kChunk records in, their results out.
+// The staging block of one GPU: two slots of kChunk records in and their
+// results out, so that an array of several chunks keeps the GPU on one slot
+// while the calling thread empties and refills the other.
 struct Staging {
   std::mutex lock;  // one call at a time per device: the block is shared
   unsigned char* host = nullptr;
   unsigned char* device = nullptr;
+  hipEvent_t filled[2] = {nullptr, nullptr};  // slot's results are in place
   uint32_t calls = 0;  // numbers the one-workgroup launches: the value they publish
 };
 constexpr size_t kOffTime = (size_t)kChunk * sizeof(hbt_kernel_record);
 constexpr size_t kOffOccOrigin = kOffTime + (size_t)kChunk * sizeof(double);
 constexpr size_t kOffOccDest = kOffOccOrigin + (size_t)kChunk * sizeof(int32_t);
 constexpr size_t kOffStatus = kOffOccDest + (size_t)kChunk * sizeof(int32_t);
-constexpr size_t kOffDone = kOffStatus + (size_t)kChunk;
+constexpr size_t kSlotBytes = (kOffStatus + (size_t)kChunk + 255) & ~(size_t)255;
+constexpr size_t kOffDone = 2 * kSlotBytes;  // one completion word for the block
 constexpr size_t kStagingBytes = kOffDone + 64;
 constexpr int kMaxDevices = 64;
 Staging g_staging[kMaxDevices];
@@ -120,16 +125,33 @@ int staging_ready(Staging& st) {
   if (st.host != nullptr) return HBT_OK;
   void* h = nullptr;
   void* d = nullptr;
+  hipEvent_t events[2] = {nullptr, nullptr};
   if (hipHostMalloc(&h, kStagingBytes, hipHostMallocDefault) != hipSuccess ||
-      hipHostGetDevicePointer(&d, h, 0) != hipSuccess || d == nullptr) {
+      hipHostGetDevicePointer(&d, h, 0) != hipSuccess || d == nullptr ||
+      hipEventCreateWithFlags(&events[0], hipEventDisableTiming) != hipSuccess ||
+      hipEventCreateWithFlags(&events[1], hipEventDisableTiming) != hipSuccess) {
     (void)hipGetLastError();
+    if (events[0] != nullptr) (void)hipEventDestroy(events[0]);
     if (h != nullptr) (void)hipHostFree(h);
     return HBT_ENOMEM;
   }
   st.host = static_cast<unsigned char*>(h);
   st.device = static_cast<unsigned char*>(d);
+  st.filled[0] = events[0];
+  st.filled[1] = events[1];
   std::memset(st.host + kOffDone, 0, 64);
   return HBT_OK;
+}
+
+// Results of `m` records from a slot to the caller's arrays at `done`.
+void copy_out(const unsigned char* slot, int64_t done, int64_t m, double* out_time_ns,
+              uint8_t* out_status, int32_t* out_occ_origin, int32_t* out_occ_dest) {
+  std::memcpy(out_time_ns + done, slot + kOffTime, (size_t)m * sizeof(double));
+  std::memcpy(out_status + done, slot + kOffStatus, (size_t)m);
+  if (out_occ_origin != nullptr)
+    std::memcpy(out_occ_origin + done, slot + kOffOccOrigin, (size_t)m * sizeof(int32_t));
+  if (out_occ_dest != nullptr)
+    std::memcpy(out_occ_dest + done, slot + kOffOccDest, (size_t)m * sizeof(int32_t));
 }
 
 // The stream must be usable for a launch followed by a wait: not under
@@ -191,43 +213,76 @@ int hbt_wave_scale_host_records(const hbt_device_spec* origin, const hbt_device_
   if ((rc = staging_ready(st)) != HBT_OK) return rc;
 
   HostRecordArgs a{};
-  a.rec = reinterpret_cast<const hbt_kernel_record*>(st.device);
-  a.time_ns = reinterpret_cast<double*>(st.device + kOffTime);
-  a.occ_origin = reinterpret_cast<int32_t*>(st.device + kOffOccOrigin);
-  a.occ_dest = reinterpret_cast<int32_t*>(st.device + kOffOccDest);
-  a.status = st.device + kOffStatus;
   a.origin = make_origin_args(*origin);
   a.dest = make_dest_args(*origin, *dest);
   const int model = dev::model_for(a.origin.dev, &a.dest, 1);
-
-  for (int64_t done = 0; done < n; done += kChunk) {
-    const int64_t m = (n - done < kChunk) ? (n - done) : kChunk;
-    std::memcpy(st.host, records + done, (size_t)m * sizeof(hbt_kernel_record));
+  const auto launch = [&](int slot, int64_t m, const dim3 grid) {
+    unsigned char* base = st.device + (size_t)slot * kSlotBytes;
     a.n = m;
-    const dim3 grid((unsigned)((m + kBlock - 1) / kBlock));
+    a.rec = reinterpret_cast<const hbt_kernel_record*>(base);
+    a.time_ns = reinterpret_cast<double*>(base + kOffTime);
+    a.occ_origin = reinterpret_cast<int32_t*>(base + kOffOccOrigin);
+    a.occ_dest = reinterpret_cast<int32_t*>(base + kOffOccDest);
+    a.status = base + kOffStatus;
+    dev::with_model(model, [&](auto mc) {
+      hipLaunchKernelGGL(wave_scale_records_kernel<decltype(mc)::value>, grid, dim3(kBlock), 0,
+                         stream, a);
+    });
+    return hipGetLastError() == hipSuccess;
+  };
+
+  if (n <= kChunk) {
+    std::memcpy(st.host, records, (size_t)n * sizeof(hbt_kernel_record));
+    const dim3 grid((unsigned)((n + kBlock - 1) / kBlock));
     // one workgroup (one kernel, a pass of a few kernels): it publishes its own
     // completion, see wait_published
     const bool publishes = grid.x == 1;
     a.done_flag = publishes ? reinterpret_cast<uint32_t*>(st.device + kOffDone) : nullptr;
     a.done_value = publishes ? ++st.calls : 0;
-    dev::with_model(model, [&](auto mc) {
-      hipLaunchKernelGGL(wave_scale_records_kernel<decltype(mc)::value>, grid, dim3(kBlock), 0,
-                         stream, a);
-    });
-    if (hipGetLastError() != hipSuccess) return HBT_EHIP;
+    if (!launch(0, n, grid)) return HBT_EHIP;
     if (!(publishes &&
           wait_published(reinterpret_cast<const uint32_t*>(st.host + kOffDone), a.done_value)) &&
         hipStreamSynchronize(stream) != hipSuccess) {
       (void)hipGetLastError();
       return HBT_EHIP;
     }
-    std::memcpy(out_time_ns + done, st.host + kOffTime, (size_t)m * sizeof(double));
-    std::memcpy(out_status + done, st.host + kOffStatus, (size_t)m);
-    if (out_occ_origin != nullptr)
-      std::memcpy(out_occ_origin + done, st.host + kOffOccOrigin, (size_t)m * sizeof(int32_t));
-    if (out_occ_dest != nullptr)
-      std::memcpy(out_occ_dest + done, st.host + kOffOccDest, (size_t)m * sizeof(int32_t));
+    copy_out(st.host, 0, n, out_time_ns, out_status, out_occ_origin, out_occ_dest);
+    return HBT_OK;
   }
+
+  // Several chunks, slots in turn: while the GPU works on one slot the calling
+  // thread copies the chunk before out of the other and, in the next turn, the
+  // next chunk into it.  A slot is refilled only after its results were taken.
+  int64_t before_done = 0, before_m = 0;  // the chunk launched one turn ago
+  int turn = 0;
+  // (an error with a launch in flight: let the stream drain before the block is used again)
+  const auto fail = [&]() {
+    (void)hipGetLastError();
+    (void)hipStreamSynchronize(stream);
+    (void)hipGetLastError();
+    return HBT_EHIP;
+  };
+  for (int64_t done = 0; done < n; done += kChunk, ++turn) {
+    const int slot = turn & 1;
+    const int64_t m = (n - done < kChunk) ? (n - done) : kChunk;
+    std::memcpy(st.host + (size_t)slot * kSlotBytes, records + done,
+                (size_t)m * sizeof(hbt_kernel_record));
+    a.done_flag = nullptr;
+    a.done_value = 0;
+    if (!launch(slot, m, dim3((unsigned)((m + kBlock - 1) / kBlock)))) return fail();
+    if (hipEventRecord(st.filled[slot], stream) != hipSuccess) return fail();
+    if (turn > 0) {
+      if (hipEventSynchronize(st.filled[slot ^ 1]) != hipSuccess) return fail();
+      copy_out(st.host + (size_t)(slot ^ 1) * kSlotBytes, before_done, before_m, out_time_ns,
+               out_status, out_occ_origin, out_occ_dest);
+    }
+    before_done = done;
+    before_m = m;
+  }
+  const int last = (turn - 1) & 1;
+  if (hipEventSynchronize(st.filled[last]) != hipSuccess) return fail();
+  copy_out(st.host + (size_t)last * kSlotBytes, before_done, before_m, out_time_ns, out_status,
+           out_occ_origin, out_occ_dest);
   return HBT_OK;
 }
 

@@ -174,10 +174,12 @@ int hbt_wave_scale(const hbt_device_spec *origin, const hbt_device_spec *dests, 
  * unless it is HBT_ST_OK.
  *
  * The records go through a pinned, device-visible staging block of the library
- * (about 1.3 MiB per GPU, allocated on the first call there and kept), in passes
- * of 16384 records; per pass one launch on `hip_stream` and a wait for the
- * stream, so the call returns with the results in place (some 15 us for up to a
- * few thousand records).  Calls on one GPU are serialised inside the library.
+ * (about 2.7 MiB per GPU, allocated on the first call there and kept): up to
+ * 16384 records in one launch on `hip_stream` and a wait, so the call returns
+ * with the results in place (some 15 us for up to a few thousand records);
+ * longer arrays in chunks of 16384 through the block's two halves in turn, one
+ * chunk on the GPU while the calling thread copies the one before out and the
+ * next in.  Calls on one GPU are serialised inside the library.
  * `hip_stream` must be a stream of the current device and must not be under
  * graph capture (HBT_EINVAL): the call waits for it.
  */

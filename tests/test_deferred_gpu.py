@@ -60,7 +60,7 @@ def call_host_records(origin, dest, records, stream=None, occupancies=True):
     return rc, t, st, oo, od
 
 
-@pytest.mark.parametrize("n", [1, 63, 257, 10_000, 16_384, 16_385, 40_000])
+@pytest.mark.parametrize("n", [1, 63, 257, 10_000, 16_384, 16_385, 40_000, 81_921])
 def test_host_records_match_the_oracle_and_the_column_kernel(n):
     """configs[0]'s records (10 000 of them among the sizes) as host structures:
     one pass through the staging block, exactly one, and three."""
