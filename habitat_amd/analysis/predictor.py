@@ -141,7 +141,12 @@ def records_from_kernels(kernels, dest_device, metadata_manager, mode="unified",
     return KernelRecords.from_numpy(rec, device=device or "cuda")
 
 
-_LAUNCH_FIELDS = operator.methodcaller("launch_fields")
+# a MeasuredKernel's launch_fields() without the two Python calls: one C-level
+# getter per kernel (kernel objects of another implementation lack these
+# names and take the AttributeError path of _fingerprint)
+_LAUNCH_FIELDS = operator.attrgetter(
+    "_c._num_blocks", "_c._block_size", "_c._dynamic_shared_memory", "_c._static_shared_memory",
+    "_c._registers_per_thread", "_c._run_time_ns")
 _RAW_METRICS = operator.attrgetter("_metrics_kernels")
 
 
