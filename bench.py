@@ -116,11 +116,16 @@ class WaveScaleCall:
 def time_steps(call, steps, warmup):
     """(wall ms per step, event ms per launch) over exactly `steps` calls."""
     import torch
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    # torch creates an event at its first record(): do that here, not inside
+    # the timed region (two creations cost some 10 us: half a microsecond per
+    # step of a 20-step run)
+    e0.record()
+    e1.record()
     for _ in range(warmup):
         call()
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
     for _ in range(steps):
