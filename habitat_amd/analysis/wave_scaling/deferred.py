@@ -42,6 +42,8 @@ RECORD_DTYPE = np.dtype([
 assert RECORD_DTYPE.itemsize == ctypes.sizeof(_lib.KernelRecord) == 64
 
 _UNIFIED, _ROOFLINE, _RESIMPLIFIED = "unified", "roofline", "resimplified"
+# A pending set is closed at this many kernels and the next call opens another.
+MAX_PENDING = 65536
 
 
 class PendingSet:
@@ -148,9 +150,10 @@ def _strategy(mode, name, doc, needs_metrics=False):
         pending = _state.pending
         if (pending is None or pending.times is not None or pending.dest is not dest_device
                 or pending.origin is not origin_device or pending.manager is not metadata_manager
-                or pending.mode is not mode):
+                or pending.mode is not mode or len(pending.kernels) >= MAX_PENDING):
             # another set begins; the one before is handed over when one of its
-            # kernels is read
+            # kernels is read (and is garbage once its results are dropped: a
+            # caller that never reads leaves at most MAX_PENDING kernels behind)
             pending = _state.pending = PendingSet(origin_device, dest_device, metadata_manager,
                                                   mode)
         kernels = pending.kernels

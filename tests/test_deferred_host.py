@@ -98,3 +98,20 @@ def test_handing_over_fails_loudly_without_a_gpu():
     p = deferred_unified_wave_scaling(kernel(), Device.V100, Device.P100, NullMetadataManager())
     with pytest.raises(RuntimeError):     # torch (no HIP GPUs) or the library (HBT_EHIP)
         p.run_time_ns
+
+
+def test_a_pending_set_is_closed_at_its_size_limit(monkeypatch):
+    """A caller that never reads its results must not make the thread's set
+    grow for ever: at MAX_PENDING kernels the set is closed and the next call
+    opens another (the closed one lives as long as its results do)."""
+    monkeypatch.setattr(deferred, "MAX_PENDING", 5)
+    mm = NullMetadataManager()
+    k = kernel()
+    results = [deferred_unified_wave_scaling(k, Device.V100, Device.P100, mm) for _ in range(12)]
+    sets = []
+    for r in results:
+        if not sets or sets[-1] is not r._set:
+            sets.append(r._set)
+    assert [len(s) for s in sets] == [5, 5, 2]
+    assert [r._index for r in results] == [0, 1, 2, 3, 4] * 2 + [0, 1]
+    assert deferred.pending_kernels() == 2
