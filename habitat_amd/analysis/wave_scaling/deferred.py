@@ -12,6 +12,8 @@ every kernel of the set has its time from then on.
 
     Predictor(wave_scaling_strategy=deferred_unified_wave_scaling)
 
+(likewise deferred_roofline_, deferred_resimplified_ and deferred_cdna_wave_scaling).
+
 What shifts against the eager strategies: the exceptions the reference raises
 inside the strategy call for a kernel that cannot be scaled
 (ZeroDivisionError, AssertionError) are raised by that kernel's `run_time_ns`
@@ -31,6 +33,7 @@ import torch
 
 from habitat_amd import _lib
 from habitat_amd.analysis.kernels import PredictedKernel, pack_record
+from habitat_amd.analysis.wave_scaling.cdna import native_description
 from habitat_amd.analysis.wave_scaling.metadata import NullMetadataManager
 from habitat_amd.analysis.wave_scaling.scalar import raise_for_status, read_metrics
 
@@ -41,7 +44,7 @@ RECORD_DTYPE = np.dtype([
     ("dram_read_bytes", "<f8"), ("dram_write_bytes", "<f8")])
 assert RECORD_DTYPE.itemsize == ctypes.sizeof(_lib.KernelRecord) == 64
 
-_UNIFIED, _ROOFLINE, _RESIMPLIFIED = "unified", "roofline", "resimplified"
+_UNIFIED, _ROOFLINE, _RESIMPLIFIED, _CDNA = "unified", "roofline", "resimplified", "cdna"
 # A pending set is closed at this many kernels and the next call opens another.
 MAX_PENDING = 65536
 
@@ -50,10 +53,16 @@ class PendingSet:
     """Kernels noted by a deferred strategy for one (origin, destination,
     metadata manager, strategy), in call order; `times` is None until the set
     has been handed to the GPU."""
-    __slots__ = ("origin", "dest", "manager", "mode", "kernels", "times", "failed")
+    __slots__ = ("origin", "dest", "manager", "mode", "kernels", "times", "failed",
+                 "model_origin", "model_dest")
 
     def __init__(self, origin, dest, manager, mode):
         self.origin, self.dest, self.manager, self.mode = origin, dest, manager, mode
+        # the descriptions whose occupancy rules apply: under the cdna strategy an
+        # AMD device's compute-unit description (the register table is still
+        # asked about the device the caller named)
+        self.model_origin = native_description(origin) if mode is _CDNA else origin
+        self.model_dest = native_description(dest) if mode is _CDNA else dest
         self.kernels = []
         self.times = None
         self.failed = None    # {index: status} of the kernels the reference raises for
@@ -92,7 +101,7 @@ class PendingSet:
         status = np.empty(n, np.uint8)
         stream = torch.cuda.current_stream()
         rc = _lib.lib().hbt_wave_scale_host_records(
-            ctypes.byref(self.origin.spec), ctypes.byref(self.dest.spec), n,
+            ctypes.byref(self.model_origin.spec), ctypes.byref(self.model_dest.spec), n,
             ctypes.c_void_p(rec.ctypes.data), ctypes.c_void_p(times.ctypes.data),
             ctypes.c_void_p(status.ctypes.data), None, None,
             ctypes.c_void_p(stream.cuda_stream))
@@ -175,6 +184,12 @@ deferred_roofline_wave_scaling = _strategy(
     _ROOFLINE, "deferred_roofline_wave_scaling",
     "roofline_wave_scaling (wave_scaling/roofline.py:8-65), deferred.  A kernel without its "
     "metrics raises AttributeError in the call, as there.", needs_metrics=True)
+
+
+deferred_cdna_wave_scaling = _strategy(
+    _CDNA, "deferred_cdna_wave_scaling",
+    "cdna_wave_scaling (unified wave scaling with AMD devices judged by the compute-unit "
+    "occupancy rules; no counterpart in the reference), deferred.")
 
 
 def pending_kernels():

@@ -240,6 +240,14 @@ def test_strategy_and_sweep_use_the_compute_unit_model():
     k = ops[0].forward.kernels[0]
     one = cdna_wave_scaling(k, Device.V100, Device.MI355X, native._kernel_metadata)
     assert one.run_time_ns == got[0].forward.kernels[0].run_time_ns
+    # the deferred form of the strategy, through the reference's loop shape: one
+    # call per kernel, times read afterwards
+    from habitat_amd.analysis.wave_scaling.deferred import deferred_cdna_wave_scaling
+    kernels = [k for op in ops for k in op.forward.kernels]
+    noted = [deferred_cdna_wave_scaling(k, Device.V100, Device.MI355X, native._kernel_metadata)
+             for k in kernels]
+    assert [p.run_time_ns for p in noted] == [
+        k.run_time_ns for o in got for k in o.forward.kernels]
     # NVIDIA to NVIDIA is untouched
     a = native.predict_operations(ops, Device.T4)
     b = dressed.predict_operations(ops, Device.T4)
